@@ -8,7 +8,8 @@ other kinds of layers, fixed-size state buffers without a length that ``reset()`
 
 * Layers whose mixers ask for the same kind of storage (an equal *need*: same kv heads, head size and window;
   or rows of the same name and shape) form a *group*.  A group has storage of its own: ``k`` and ``v`` of shape
-  ``[layers of the group, pages + 1, kv_heads, PAGE_TOKENS, head_dim]`` (``v`` with the last two swapped) and one page table (the pages
+  ``[layers of the group, pages + 1, kv_heads, PAGE_TOKENS, head_dim]`` (``v`` with the last two swapped, and with a
+  head count and size of its own if the need says so) and one page table (the pages
   of every slot), shared by the group's layers.  The last page is never handed out: rows that pad a
   batch write there.
 * State groups are ``[layers of the group, slots + 1, *shape]``, zeroed when a slot is opened.
@@ -46,6 +47,10 @@ class KVNeed:
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    # a mixer whose keys and values differ in count or size (several key rows for one value row, a value size of
+    # its own) says so; None: as many value heads as key heads, of the keys' size
+    value_heads: int | None = None
+    value_dim: int | None = None
 
     def make_group(self, n_entries, n_pages, n_slots, max_pages_per_slot, dtype, device):
         return KVGroup(self, n_entries, n_pages, n_slots, max_pages_per_slot, dtype, device)
@@ -134,11 +139,11 @@ class KVGroup(PagedGroup):
         # index that is contiguous in memory
         self.k = torch.zeros((n_entries, n_pages + 1, need.num_kv_heads, PAGE_TOKENS, need.head_dim), dtype=dtype,
                              device=device)
-        self.v = torch.zeros((n_entries, n_pages + 1, need.num_kv_heads, need.head_dim, PAGE_TOKENS), dtype=dtype,
-                             device=device)
+        self.v = torch.zeros((n_entries, n_pages + 1, need.value_heads or need.num_kv_heads, need.value_dim or need.head_dim,
+                              PAGE_TOKENS), dtype=dtype, device=device)
 
     def nbytes(self) -> int:
-        return 2 * self.k.numel() * self.k.element_size()
+        return (self.k.numel() + self.v.numel()) * self.k.element_size()
 
     def attach(self, layer_cache, entry: int) -> None:
         if layer_cache.kv is not None:

@@ -37,6 +37,8 @@ def registered_architectures() -> list[str]:
 
 def config_class_for(raw: dict) -> type:
     archs = raw.get("architectures") or []
+    if not archs and isinstance(raw.get("architecture"), str):       # some configurations name one, in the singular
+        archs = [raw["architecture"]]
     for a in archs:
         if a in _BY_ARCHITECTURE:
             return _BY_ARCHITECTURE[a]

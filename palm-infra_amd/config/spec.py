@@ -137,6 +137,8 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     stop_token_ids: tuple[int, ...] = ()
+    # layers read the results of all layers before them (and the embedding's rows): the model keeps them for the step
+    keeps_results: bool = False
 
     def __post_init__(self):
         for i, call in enumerate(self.order):

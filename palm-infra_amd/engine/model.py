@@ -45,7 +45,13 @@ class DecoderModel:
     def forward(self, ctx, cache, want_rows: torch.Tensor | None) -> torch.Tensor:
         """Run the step's tokens through all layers; logits (float32) at the rows ``want_rows`` of the
         packed tokens (all rows if None)."""
-        x = self.embedding.forward(ctx.token_ids)
+        if self.spec.keeps_results and self.order:
+            # layers read earlier layers' results: plane 0 holds the embedding rows, plane i + 1 the i-th run's result
+            ctx.results = torch.empty((len(self.order) + 1, ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32,
+                                      device=self.device)
+            x = self.embedding.forward(ctx.token_ids, out=ctx.results[0]).clone()
+        else:
+            x = self.embedding.forward(ctx.token_ids)
         if not self.order:
             return self.head.forward(self.final_norm(x, rows=want_rows))
         # a layer gets its first norm's output and returns the output of the norm after it: the next layer's
@@ -59,4 +65,5 @@ class DecoderModel:
                 sink = ResidualSink(x, self.final_norm, rows=want_rows)
             h = self.layers[call.layer].forward(x, h, ctx, sink)
         ctx.layer_cache = None
+        ctx.results = None
         return self.head.forward(h)

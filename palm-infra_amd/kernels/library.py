@@ -9,6 +9,9 @@ built or loaded, the error says so and nothing runs.
 Libraries:
   ``core``              every kernel that does not depend on the head size
   ``attention_hd<N>``   the matrix-core attention kernels, compiled for one head size
+  ``mixers``            the mixers beside softmax attention over equal key and value sizes (retention, the selective
+                        scan and its convolution, differential attention) and the stream of blocks that norm a
+                        branch's output; loaded when a model has such a part
 """
 from __future__ import annotations
 
@@ -38,6 +41,7 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
                 "linear_wide_gated_32.hip", "linear_wide_gated_64.hip", "linear_wide_store_128.hip", "linear_wide_gated_128.hip", "linear_mid.hip",
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
+MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
 
@@ -163,6 +167,8 @@ def _compile(name: str, sources, defines, force: bool) -> Path:
 def _spec(name: str):
     if name == "core":
         return CORE_SOURCES, ()
+    if name == "mixers":
+        return MIXER_SOURCES, ()
     if name.startswith("attention_hd"):
         hd = int(name[len("attention_hd"):])
         return ATTENTION_SOURCES, (f"PALM_HEAD_DIM={hd}",)

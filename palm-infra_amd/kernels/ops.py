@@ -753,3 +753,190 @@ def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int,
                                  ctx.max_new, nh, nkv, hd, scale, window)
     return attention_exact(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,
                            ctx.max_new, nh, nkv, hd, scale, window)
+
+
+# ---- mixers beside softmax attention, and blocks that norm a branch's output (library ``mixers``) -----------------
+
+_MIXER_SIGNATURES = {
+    "palm_add_normed": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p, c_int,
+                        c_longlong, c_void_p, c_int],
+    "palm_xielu": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_longlong],
+    "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                       c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "palm_causal_conv": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                         c_int, c_int, c_int, c_void_p],
+    "palm_selective_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "palm_diff_qkv_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                            c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_int],
+    "palm_attention_diff": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p],
+}
+_mixers = None
+
+
+def mixers():
+    """The library of the other mixers' kernels, with the argument types of its entry points declared."""
+    global _mixers
+    if _mixers is None:
+        lib = library.load("mixers")
+        for name, argtypes in _MIXER_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = argtypes, c_int
+        _mixers = lib
+    return _mixers
+
+
+def add_normed(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+               results: torch.Tensor | None = None, mix: torch.Tensor | None = None) -> torch.Tensor:
+    """x += delta / sqrt(mean(delta^2) + eps) * weight, row by row, in place (x float32 [n, width]).
+
+    ``results`` float32 [P, n, width] with ``mix`` float32 [J + 1], J < P: the sum is also written to plane J, and x
+    becomes sum_j mix[j] * results[j], j = 0 .. J (the planes below J hold earlier layers' results).
+
+    Returns x in ``out_dtype`` for the branch that reads it next: x itself if that is float32, else a rounded copy
+    made in the same pass."""
+    _dev("add_normed", x, delta, weight, results, mix)
+    _need(x.dim() == 2 and x.dtype == F32 and delta.shape == x.shape, f"add_normed: x {tuple(x.shape)} {x.dtype}, delta {tuple(delta.shape)}")
+    n, width = x.shape
+    _need(weight.shape == (width,) and weight.dtype == F32, f"add_normed: the norm's weight is float32 [{width}]")
+    planes, stride = 0, 0
+    if results is not None:
+        _need(mix is not None and mix.dtype == F32 and mix.dim() == 1 and results.dtype == F32 and results.dim() == 3
+              and results.shape[1:] == x.shape and 1 <= mix.shape[0] <= results.shape[0],
+              f"add_normed: results {tuple(results.shape)} {results.dtype} and {None if mix is None else tuple(mix.shape)} weights")
+        planes, stride = mix.shape[0], n * width
+    else:
+        _need(mix is None, "add_normed: weights without results")
+    out = x if out_dtype == F32 else torch.empty((n, width), dtype=out_dtype, device=x.device)
+    library.call(mixers(), "palm_add_normed", _stream(), _p(x), _p(delta), _code(delta, "add_normed delta"), _p(weight), float(eps),
+                 n, width, _p(results), _p(mix), planes, stride, None if out is x else _p(out), _code(out, "add_normed out"))
+    return out
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    """z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2, with pq = [p, q] float32."""
+    _dev("xielu", z, pq)
+    _need(pq.shape == (2,) and pq.dtype == F32, f"xielu: the two numbers are float32 [2], not {pq.dtype} {tuple(pq.shape)}")
+    out = torch.empty_like(z)
+    library.call(mixers(), "palm_xielu", _stream(), _p(z), _p(out), _code(z, "xielu"), _p(pq), z.numel())
+    return out
+
+
+def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, k_scale: float, eps: float,
+              state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0) -> torch.Tensor:
+    """The step's tokens through a retention layer's recurrence.  qkvg [n, heads * (2 dim + 2 vdim)] holds q | k | v |
+    gate; state float32 [slots, heads, dim, vdim] is read and left updated.  Returns [n, heads * vdim]: the heads'
+    outputs, unit-normed per head and gated."""
+    _dev("retention", qkvg, decay, state, cos, sin, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    _i32("retention", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    n = qkvg.shape[0]
+    _need(qkvg.dim() == 2 and qkvg.shape[1] == heads * (2 * dim + 2 * vdim), f"retention: rows {tuple(qkvg.shape)} are not "
+          f"[n, {heads} * (2*{dim} + 2*{vdim})]")
+    _need(decay.shape == (heads,) and decay.dtype == F32, f"retention: one float32 decay for each of {heads} heads")
+    _need(state.dim() == 4 and state.shape[1:] == (heads, dim, vdim) and state.dtype == F32,
+          f"retention: state {tuple(state.shape)} {state.dtype} is not float32 [slots, {heads}, {dim}, {vdim}]")
+    _need(n == ctx.n_tokens, "retention: one row for each token of the step")
+    if rot:
+        for tab in (cos, sin):
+            _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"retention: rotation rows are float32 [{n}, {rot // 2}]")
+    out = torch.empty((n, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    library.call(mixers(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
+                 2 * heads * dim, 2 * heads * dim + heads * vdim, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
+                 _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out))
+    return out
+
+
+def causal_conv(xz: torch.Tensor, channels: int, weight: torch.Tensor, bias: torch.Tensor, conv_state: torch.Tensor, ctx) -> torch.Tensor:
+    """silu(bias + a causal convolution per channel) over the first ``channels`` columns of xz [n, >= channels];
+    weight float32 [channels, taps] (last column: the current token), conv_state float32 [slots, taps - 1, channels]:
+    each sequence's last inputs, read and left updated."""
+    _dev("causal_conv", xz, weight, bias, conv_state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    _i32("causal_conv", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    taps = weight.shape[1]
+    _need(xz.dim() == 2 and xz.shape[1] >= channels and xz.shape[0] == ctx.n_tokens, f"causal_conv: input {tuple(xz.shape)}")
+    _need(weight.shape == (channels, taps) and weight.dtype == F32 and bias.shape == (channels,) and bias.dtype == F32,
+          f"causal_conv: weight {tuple(weight.shape)} {weight.dtype}, bias {tuple(bias.shape)} {bias.dtype}")
+    _need(conv_state.dim() == 3 and conv_state.shape[1:] == (max(taps - 1, 0), channels) and conv_state.dtype == F32,
+          f"causal_conv: state {tuple(conv_state.shape)} is not float32 [slots, {taps - 1}, {channels}]")
+    out = torch.empty((xz.shape[0], channels), dtype=xz.dtype, device=xz.device)
+    library.call(mixers(), "palm_causal_conv", _stream(), _p(xz), _code(xz, "causal_conv"), xz.shape[1], _p(weight), _p(bias),
+                 _p(conv_state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, ctx.max_new, channels, taps, _p(out))
+    return out
+
+
+def selective_scan(u: torch.Tensor, xz: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, dt_linear: torch.Tensor,
+                   dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, ctx) -> torch.Tensor:
+    """u [n, C] (the convolution's output), the gate z = xz[:, C:2C], B = bc[:, b_off:b_off+N], C = bc[:, c_off:c_off+N],
+    dt_linear float32 [n, C] (before bias and softplus), a_log float32 [C, N], state float32 [slots, C, N] read and
+    left updated.  Returns y * silu(z), [n, C]."""
+    _dev("selective_scan", u, xz, bc, dt_linear, dt_bias, a_log, d_skip, state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    _i32("selective_scan", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    n, C = u.shape
+    N = a_log.shape[1]
+    _need(xz.shape == (n, 2 * C) and xz.dtype == u.dtype and bc.dtype == u.dtype and bc.dim() == 2 and bc.shape[0] == n
+          and 0 <= b_off and b_off + N <= bc.shape[1] and 0 <= c_off and c_off + N <= bc.shape[1],
+          f"selective_scan: u {tuple(u.shape)}, xz {tuple(xz.shape)}, bc {tuple(bc.shape)}")
+    _need(dt_linear.shape == (n, C) and dt_linear.dtype == F32, f"selective_scan: step sizes {tuple(dt_linear.shape)} {dt_linear.dtype} are float32 [{n}, {C}]")
+    for v, nm in ((dt_bias, "dt bias"), (d_skip, "D")):
+        _need(v.shape == (C,) and v.dtype == F32, f"selective_scan: {nm} is float32 [{C}]")
+    _need(a_log.shape == (C, N) and a_log.dtype == F32, f"selective_scan: A_log {tuple(a_log.shape)} {a_log.dtype}")
+    _need(state.dim() == 3 and state.shape[1:] == (C, N) and state.dtype == F32, f"selective_scan: state {tuple(state.shape)} {state.dtype}")
+    _need(n == ctx.n_tokens, "selective_scan: one row for each token of the step")
+    out = torch.empty((n, C), dtype=u.dtype, device=u.device)
+    library.call(mixers(), "palm_selective_scan", _stream(), _p(u), xz.data_ptr() + C * xz.element_size(), 2 * C, _p(bc), bc.shape[1],
+                 int(b_off), int(c_off), _code(u, "selective_scan"), _p(dt_linear), _p(dt_bias), _p(a_log), _p(d_skip), _p(state),
+                 _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, C, N, _p(out))
+    return out
+
+
+def _check_diff_cache(what, k_cache, v_cache, block_table, kv_heads, dim, vdim):
+    _need(k_cache.dim() == 4 and k_cache.shape[1:] == (2 * kv_heads, PAGE_TOKENS, dim),
+          f"{what}: key cache {tuple(k_cache.shape)} is not [pages, 2*{kv_heads}, {PAGE_TOKENS}, {dim}]")
+    _need(v_cache.shape == (k_cache.shape[0], kv_heads, vdim, PAGE_TOKENS) and v_cache.dtype == k_cache.dtype,
+          f"{what}: value cache {tuple(v_cache.shape)} is not [pages, {kv_heads}, {vdim}, {PAGE_TOKENS}]")
+    _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
+
+
+def diff_qkv_store(qkv: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, q_norm_w, k_norm_w, eps: float,
+                   k_cache, v_cache, block_table, ctx, write_cache: bool = True) -> torch.Tensor:
+    """qkv [n, 2 heads dim + 2 kv_heads dim + kv_heads vdim] -> q [n, 2 heads dim], RMS-normed per head and map; k
+    (normed likewise) and v go to the cache page of each token."""
+    what = "diff_qkv_store"
+    _dev(what, qkv, q_norm_w, k_norm_w, k_cache, v_cache, block_table, ctx.tok_slot, ctx.positions)
+    _i32(what, block_table, ctx.tok_slot, ctx.positions)
+    n = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == 2 * (heads + kv_heads) * dim + kv_heads * vdim, f"{what}: rows {tuple(qkv.shape)}")
+    for w in (q_norm_w, k_norm_w):
+        _need(w.shape == (dim,) and w.dtype == F32, f"{what}: a norm weight is float32 [{dim}]")
+    _check_diff_cache(what, k_cache, v_cache, block_table, kv_heads, dim, vdim)
+    _need(k_cache.dtype == qkv.dtype, f"{what}: cache is {k_cache.dtype}, activations are {qkv.dtype}")
+    _need(n == ctx.n_tokens, f"{what}: one row for each token of the step")
+    q = torch.empty((n, 2 * heads * dim), dtype=qkv.dtype, device=qkv.device)
+    library.call(mixers(), "palm_diff_qkv_store", _stream(), _p(qkv), _code(qkv, what), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(ctx.tok_slot), _p(ctx.positions), _p(q_norm_w), _p(k_norm_w), float(eps), n, heads, kv_heads,
+                 dim, vdim, int(write_cache))
+    return q
+
+
+def attention_diff_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
+                         scale: float, lam: float, gain: float, eps: float) -> torch.Tensor:
+    """Differential attention of the step's queries over the cache in 32-bit arithmetic: out [n, heads * vdim] =
+    unit_rms(a1 - lam * a2) * gain per head."""
+    what = "attention_diff"
+    _dev(what, q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    n = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == 2 * heads * dim and n == ctx.n_tokens, f"{what}: q {tuple(q.shape)} is not [n, 2*{heads}*{dim}]")
+    _check_diff_cache(what, k_cache, v_cache, block_table, kv_heads, dim, vdim)
+    _need(k_cache.dtype == q.dtype, f"{what}: cache is {k_cache.dtype}, queries are {q.dtype}")
+    out = torch.empty((n, heads * vdim), dtype=q.dtype, device=q.device)
+    library.call(mixers(), "palm_attention_diff", _stream(), _p(q), _code(q, what), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
+                 heads, kv_heads, dim, vdim, float(scale), float(lam), float(gain), float(eps), _p(out))
+    return out
+
+
+def attention_diff(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps):
+    """The step's queries over the cache; picks the kernel by element type and step shape."""
+    return attention_diff_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps)

@@ -96,6 +96,7 @@ class StepContext:
     is_decode: bool = False      # every sequence brings exactly one token
     decode_slices: int = 0       # if set: into how many slices decode attention cuts a key range (else chosen per call)
     layer_cache: object = None   # the LayerCache of the run-order entry that is running
+    results: object = None       # float32 [planes, n, width] if the model keeps every layer's result for later layers to read
     memo: dict = field(default_factory=dict)   # what parts make once per step (rotation tables)
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host
 

@@ -6,11 +6,19 @@ stream x is float32.  A branch's output is never added by a kernel of its own: i
 norms (the sum is made in 32-bit and written back to x), or the branch's last product does both.  So the
 block gets its first norm's output from whoever ran before it, and returns the output of the norm that comes
 after it.
+
+``post_norm``: x += norm(mixer(x)); x += norm(feed_forward(x)): the norm sits on each branch's output, and the
+branches read the stream itself (in the activation type).  A layer may have no feed-forward.  With
+``depth_weights`` c (float32 [J + 1]) the layer's result R_J = x is kept beside the earlier ones (R_0: the embedding
+rows) and what goes on is sum_j c[j] R_j: the model must say ``keeps_results``.  The norm, the add, the average and
+the rounded copy for the next reader are one kernel.
 """
 from __future__ import annotations
 
+from ..kernels import ops
 from .base import cache_needs, register_part
-from .residual import ResidualSink, run_branch
+from .norm import PassThrough
+from .residual import ResidualSink, as_tensor, run_branch
 
 
 @register_part("block", "pre_norm")
@@ -37,3 +45,48 @@ class PreNormBlock:
     def forward(self, x, h, ctx, sink):
         h = run_branch(self.mixer, h, ctx, ResidualSink(x, self.feed_forward_norm))
         return run_branch(self.feed_forward, h, ctx, sink)
+
+
+@register_part("block", "post_norm")
+class PostNormBlock:
+    def __init__(self, spec, builder):
+        self.mixer = builder.build(spec.parts["mixer"])
+        self.mixer_norm = builder.build(spec.parts["mixer_norm"])
+        self.feed_forward = builder.build(spec.parts["feed_forward"]) if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"]) if self.feed_forward is not None else None
+        self.depth_weights = builder.tensor(spec, "depth_weights") if "depth_weights" in spec.tensors else None
+        self.dtype = builder.dtype
+        self._reader = PassThrough(dtype=builder.dtype)
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and not getattr(norm, "folds_into_products", False):
+                raise ValueError("a post_norm block norms its branches' outputs with RMS norms")
+
+    @property
+    def capturable(self) -> bool:
+        parts = [self.mixer, self.mixer_norm] + ([self.feed_forward, self.feed_forward_norm] if self.feed_forward else [])
+        return all(getattr(p, "capturable", False) for p in parts)
+
+    @staticmethod
+    def cache_needs(spec):
+        return cache_needs(spec.parts["mixer"])
+
+    @property
+    def entry_norm(self):
+        return self._reader
+
+    def forward(self, x, h, ctx, sink):
+        branches = [(self.mixer, self.mixer_norm)]
+        if self.feed_forward is not None:
+            branches.append((self.feed_forward, self.feed_forward_norm))
+        for i, (part, norm) in enumerate(branches):
+            y = part.forward(as_tensor(h), ctx)
+            last = i + 1 == len(branches)
+            if last and self.depth_weights is not None:
+                if ctx.results is None:
+                    raise RuntimeError("a block that averages over depth needs the earlier layers' results; the model keeps none")
+                h = ops.add_normed(x, y, norm.weight, norm.eps, self.dtype, results=ctx.results, mix=self.depth_weights)
+            else:
+                h = ops.add_normed(x, y, norm.weight, norm.eps, self.dtype)
+        if sink.rows is None and getattr(sink.norm, "passes_through", False):
+            return h                                        # the next block reads the stream as it is
+        return sink.norm(sink.x, rows=sink.rows)

@@ -21,8 +21,8 @@ class TokenEmbedding:
         if self.table.shape != (self.vocab, self.hidden):
             raise ValueError(f"embedding table {tuple(self.table.shape)} is not [{self.vocab}, {self.hidden}]")
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        return ops.embed(self.table, token_ids)
+    def forward(self, token_ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        return ops.embed(self.table, token_ids, out)
 
 
 @register_part("head", "linear")

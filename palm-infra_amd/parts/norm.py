@@ -26,3 +26,32 @@ class RMSNorm:
     def __call__(self, x: torch.Tensor, delta: torch.Tensor | None = None, update: bool = False,
                  rows: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
         return ops.rmsnorm(x, self.weight, self.eps, out_dtype or self.dtype, delta=delta, update_x=update, rows=rows)
+
+
+@register_part("norm", "none")
+class PassThrough:
+    """No norm at all, for blocks whose branches read the residual stream itself: the rows (plus ``delta``) in the
+    activation type.  In the float32 mode, without a delta or a row selection, that is the stream itself."""
+    capturable = True
+    passes_through = True
+
+    def __init__(self, spec=None, builder=None, dtype: torch.dtype | None = None):
+        self.dtype = dtype if dtype is not None else builder.dtype
+
+    def __call__(self, x: torch.Tensor, delta: torch.Tensor | None = None, update: bool = False,
+                 rows: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        out_dtype = out_dtype or self.dtype
+        if delta is not None:
+            if delta.dim() == 3:
+                delta = delta.sum(0)
+            total = x + delta.to(torch.float32)
+            if update:
+                x.copy_(total)
+            x = total
+        if rows is not None:
+            x = x.index_select(0, rows.long())
+        if out_dtype == x.dtype:
+            return x
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        ops.convert_into(x, out)
+        return out
