@@ -111,8 +111,10 @@ def retention(h, w, pre, m, eps):
     q = (h @ w[pre + "q"].T).view(T, H, d)
     k = (h @ w[pre + "k"].T).view(T, H, d)
     v = (h @ w[pre + "v"].T).view(T, H, dv)
-    q = rotate_half_split(q, m["rot"]["dims"], m["rot"]["base"])
-    k = rotate_half_split(k, m["rot"]["dims"], m["rot"]["base"]) * d ** -0.5
+    if m.get("rot"):
+        q = rotate_half_split(q, m["rot"]["dims"], m["rot"]["base"])
+        k = rotate_half_split(k, m["rot"]["dims"], m["rot"]["base"])
+    k = k * d ** -0.5
     out = torch.zeros(T, H, dv, dtype=F64)
     for hd in range(H):
         S = torch.zeros(d, dv, dtype=F64)
