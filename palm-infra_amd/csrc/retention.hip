@@ -12,12 +12,21 @@
 // q and k into LDS, every thread then does its column's updates and dot products for the tile's tokens, and the
 // per-token sums of squares over v are reduced for the whole tile at once.  A prompt and a single token run
 // the same code, so a prompt leaves the state that its tokens one by one leave.
+//
+// A long run of new tokens would keep only (heads x sequences) blocks busy, one after the other token.  Such a run is
+// cut into chunks of `chunk` tokens, and the recurrence's linearity does the rest in three launches:
+//   1. every chunk alone from a zero state: its own sum  L_c = sum_t g^(end - t) k_t v_t^T         (all chunks at once)
+//   2. the chunks' starting states, one after the other: S_(c+1) = g^len_c S_c + L_c, S_0 the kept state   (elementwise)
+//   3. every chunk from its starting state, now with outputs                                        (all chunks at once)
+// The arithmetic of a token is the same in all three; only the order of the 32-bit sums over the past differs.
 #include "common.h"
 
 constexpr int RET_TILE = 8;
 
+enum RetentionMode : int { RET_WHOLE = 0, RET_LOCAL = 1, RET_FROM_STARTS = 2 };
+
 template <typename T, int DMAX>
-__global__ void retention_kernel(const T* __restrict__ qkvg, int row_stride, int q_off, int k_off, int v_off, int g_off,
+__global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, const T* __restrict__ qkvg, int row_stride, int q_off, int k_off, int v_off, int g_off,
                                  const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
                                  const float* __restrict__ decay, float k_scale, float eps,
                                  float* __restrict__ state, const int* __restrict__ seq_slot,
@@ -25,18 +34,23 @@ __global__ void retention_kernel(const T* __restrict__ qkvg, int row_stride, int
                                  int heads, int dim, int vdim, T* __restrict__ out) {
     __shared__ float q_s[RET_TILE][DMAX], k_s[RET_TILE][DMAX];
     __shared__ float red[RET_TILE][16];
-    const int h = blockIdx.x, b = blockIdx.y;
+    const int h = blockIdx.x, b = blockIdx.y / max_chunks, c = blockIdx.y % max_chunks;
     const int v = threadIdx.x;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
-    const int n_new = seq_new[b], row0 = cu_new[b];
+    // this block's run of tokens: the sequence's new ones, or one chunk of them
+    const int seq_tokens = seq_new[b];
+    if (c * chunk >= seq_tokens) return;
+    const int n_new = mode == RET_WHOLE ? seq_tokens : min(chunk, seq_tokens - c * chunk);
+    const int row0 = cu_new[b] + (mode == RET_WHOLE ? 0 : c * chunk);
     const bool mine = v < vdim;
     const float g = decay[h];
     const int half = rot / 2;
-    float* sp = state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + v;
+    float* sp = mode == RET_WHOLE ? state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + v
+                                  : starts + ((((size_t)b * max_chunks + c) * heads + h) * dim) * vdim + v;
 
     float S[DMAX];
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) S[d] = (mine && d < dim) ? sp[(size_t)d * vdim] : 0.f;
+    for (int d = 0; d < DMAX; ++d) S[d] = (mine && d < dim && mode != RET_LOCAL) ? sp[(size_t)d * vdim] : 0.f;
 
     for (int t0 = 0; t0 < n_new; t0 += RET_TILE) {
         const int tt = min(RET_TILE, n_new - t0);
@@ -76,13 +90,15 @@ __global__ void retention_kernel(const T* __restrict__ qkvg, int row_stride, int
                 }
                 o[ti] = acc;
             }
-            const float ss = wave_sum(o[ti] * o[ti]);
-            if (lane == 0) red[ti][wave] = ss;
+            if (mode != RET_LOCAL) {
+                const float ss = wave_sum(o[ti] * o[ti]);
+                if (lane == 0) red[ti][wave] = ss;
+            }
         }
         __syncthreads();
 #pragma unroll
         for (int ti = 0; ti < RET_TILE; ++ti) {
-            if (ti < tt && mine) {
+            if (ti < tt && mine && mode != RET_LOCAL) {
                 float total = 0.f;
                 for (int w = 0; w < n_waves; ++w) total += red[ti][w];
                 const float inv = 1.0f / sqrtf(total / (float)vdim + eps);
@@ -93,45 +109,81 @@ __global__ void retention_kernel(const T* __restrict__ qkvg, int row_stride, int
         }
         __syncthreads();
     }
-    if (mine && n_new > 0) {
+    if (mine && n_new > 0 && mode != RET_FROM_STARTS) {
 #pragma unroll
         for (int d = 0; d < DMAX; ++d)
             if (d < dim) sp[(size_t)d * vdim] = S[d];
     }
 }
 
+// Step 2 above: one thread per element of (sequence, head, dim, vdim).  starts[b][c] holds L_c and leaves as S_c.
+__global__ void retention_starts_kernel(float* __restrict__ starts, float* __restrict__ state, const float* __restrict__ decay,
+                                        const int* __restrict__ seq_slot, const int* __restrict__ seq_new, int chunk,
+                                        int max_chunks, int heads, int per_head) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (e >= heads * per_head) return;
+    const int n_new = seq_new[b];
+    if (n_new <= 0) return;
+    const float g = decay[e / per_head];
+    float* st = state + (size_t)seq_slot[b] * heads * per_head + e;
+    float s = *st;
+    for (int c = 0; c * chunk < n_new; ++c) {
+        float* at = starts + ((size_t)b * max_chunks + c) * heads * per_head + e;
+        const float local = *at;
+        *at = s;
+        s = fmaf(powf(g, (float)min(chunk, n_new - c * chunk)), s, local);
+    }
+    *st = s;
+}
+
 template <typename T>
-static int retention_launch(hipStream_t stream, dim3 grid, int threads, const T* qkvg, int row_stride, int q_off, int k_off,
-                            int v_off, int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay,
-                            float k_scale, float eps, float* state, const int* seq_slot, const int* seq_new,
-                            const int* cu_new, int heads, int dim, int vdim, T* out) {
-#define RET_CASE(D) retention_kernel<T, D><<<grid, threads, 0, stream>>>(qkvg, row_stride, q_off, k_off, v_off, g_off, cos_t, \
-        sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out)
-    if (dim <= 16) RET_CASE(16);
-    else if (dim <= 32) RET_CASE(32);
+static void retention_launch(hipStream_t stream, dim3 grid, int threads, int mode, int chunk, int max_chunks, float* starts,
+                             const T* qkvg, int row_stride, int q_off, int k_off,
+                             int v_off, int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay,
+                             float k_scale, float eps, float* state, const int* seq_slot, const int* seq_new,
+                             const int* cu_new, int heads, int dim, int vdim, T* out) {
+#define RET_CASE(D) retention_kernel<T, D><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, row_stride, q_off, k_off, \
+        v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out)
+    if (dim <= 32) RET_CASE(32);
     else if (dim <= 64) RET_CASE(64);
     else if (dim <= 128) RET_CASE(128);
     else RET_CASE(256);
 #undef RET_CASE
-    return 0;
 }
 
+// chunk == 0: every sequence's run in one block per head.  Else `starts` holds n_seqs * max_chunks * heads * dim * vdim
+// floats, max_chunks = ceil(max_new / chunk).
 PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int row_stride, int q_off, int k_off, int v_off,
                             int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay, float k_scale,
                             float eps, float* state, const int* seq_slot, const int* seq_new, const int* cu_new, int n_seqs,
-                            int heads, int dim, int vdim, void* out) {
+                            int heads, int dim, int vdim, void* out, int max_new, int chunk, float* starts) {
     PALM_CHECK(n_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0, "retention: seqs=%d heads=%d dim=%d vdim=%d", n_seqs, heads, dim, vdim);
     PALM_CHECK(dim <= 256, "retention: a key size of %d exceeds 256", dim);
     PALM_CHECK(vdim <= 1024, "retention: a value size of %d exceeds 1024", vdim);
     PALM_CHECK(rot >= 0 && rot <= dim && rot % 2 == 0, "retention: %d rotated dimensions of %d", rot, dim);
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "retention: a rotation needs its cos and sin rows");
-    PALM_CHECK(heads <= 65535 && n_seqs <= 65535, "retention: %d heads / %d sequences are more than one launch takes", heads, n_seqs);
+    PALM_CHECK(chunk >= 0 && (chunk == 0 || (starts && max_new > 0)), "retention: chunks of %d tokens need their starting states", chunk);
     if (n_seqs == 0) return 0;
+    const int max_chunks = chunk > 0 ? (max_new + chunk - 1) / chunk : 1;
+    PALM_CHECK(heads <= 65535 && (long long)n_seqs * max_chunks <= 65535, "retention: %d heads / %d sequences x %d chunks are more than one launch takes",
+               heads, n_seqs, max_chunks);
     const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
-    dim3 grid(heads, n_seqs);
-    PALM_DTYPE_SWITCH(dtype, T,
-        retention_launch<T>(stream, grid, threads, (const T*)qkvg, row_stride, q_off, k_off, v_off, g_off, cos_t, sin_t, rot,
-                            decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out));
+    dim3 grid(heads, n_seqs * max_chunks);
+    PALM_DTYPE_SWITCH(dtype, T, {
+        if (chunk == 0) {
+            retention_launch<T>(stream, grid, threads, RET_WHOLE, 1 << 30, 1, nullptr, (const T*)qkvg, row_stride, q_off, k_off, v_off,
+                                g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+        } else {
+            retention_launch<T>(stream, grid, threads, RET_LOCAL, chunk, max_chunks, starts, (const T*)qkvg, row_stride, q_off, k_off,
+                                v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+            const int elems = heads * dim * vdim;
+            retention_starts_kernel<<<dim3((elems + 255) / 256, n_seqs), 256, 0, stream>>>(starts, state, decay, seq_slot, seq_new, chunk,
+                                                                                         max_chunks, heads, dim * vdim);
+            retention_launch<T>(stream, grid, threads, RET_FROM_STARTS, chunk, max_chunks, starts, (const T*)qkvg, row_stride, q_off,
+                                k_off, v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim,
+                                vdim, (T*)out);
+        }
+    });
     PALM_LAUNCHED();
     return 0;
 }

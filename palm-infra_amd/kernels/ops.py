@@ -762,7 +762,8 @@ _MIXER_SIGNATURES = {
                         c_longlong, c_void_p, c_int],
     "palm_xielu": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_longlong],
     "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
-                       c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                       c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
+                       c_void_p],
     "palm_causal_conv": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_void_p],
     "palm_selective_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -823,11 +824,27 @@ def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
     return out
 
 
+RETENTION_BLOCKS_WANTED = 512      # a long run of new tokens is cut into chunks until about this many blocks run
+RETENTION_MIN_CHUNK = 32
+
+
+def retention_chunk(n_seqs: int, heads: int, max_new: int) -> int:
+    """Into chunks of how many tokens the retention kernel cuts the step's runs of new tokens (0: not at all).  One
+    block per (head, sequence) walks over its tokens one after the other; where that leaves most of the chip idle and
+    the runs are long, chunks run side by side at the price of walking over every token twice."""
+    per_seq = RETENTION_BLOCKS_WANTED // max(1, heads * n_seqs)
+    if max_new <= 2 * RETENTION_MIN_CHUNK or per_seq <= 1:
+        return 0
+    chunk = max(RETENTION_MIN_CHUNK, -(-max_new // per_seq))
+    chunk = (chunk + 7) // 8 * 8
+    return chunk if chunk < max_new else 0
+
+
 def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, k_scale: float, eps: float,
-              state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0) -> torch.Tensor:
+              state: torch.Tensor, ctx, cos=None, sin=None, rot: int = 0, chunk: int | None = None) -> torch.Tensor:
     """The step's tokens through a retention layer's recurrence.  qkvg [n, heads * (2 dim + 2 vdim)] holds q | k | v |
     gate; state float32 [slots, heads, dim, vdim] is read and left updated.  Returns [n, heads * vdim]: the heads'
-    outputs, unit-normed per head and gated."""
+    outputs, unit-normed per head and gated.  ``chunk``: see ``retention_chunk`` (None: chosen here)."""
     _dev("retention", qkvg, decay, state, cos, sin, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     _i32("retention", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     n = qkvg.shape[0]
@@ -841,9 +858,15 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
         for tab in (cos, sin):
             _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"retention: rotation rows are float32 [{n}, {rot // 2}]")
     out = torch.empty((n, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    chunk = retention_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
+    starts = None
+    if chunk:
+        max_chunks = -(-ctx.max_new // chunk)
+        starts = torch.empty((ctx.n_seqs * max_chunks, heads, dim, vdim), dtype=F32, device=qkvg.device)
     library.call(mixers(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
                  2 * heads * dim, 2 * heads * dim + heads * vdim, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
-                 _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out))
+                 _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out),
+                 int(ctx.max_new), chunk, _p(starts))
     return out
 
 

@@ -255,16 +255,21 @@ def test_retention_kernel_keeps_a_far_token_and_forgets_at_its_decay(dtype):
     without = o[T - 1, 0] - 0.99 ** (T - 1 - far) * (q[T - 1, 0] @ k[far, 0]) * v[far, 0]
     assert without.norm() < 0.3 * o[T - 1, 0].norm()
     tol = 2e-5 if dtype == torch.float32 else 3e-2
-    for portion in (T, 64, 5, 2):
+    final = None
+    # (tokens a step, tokens a chunk inside the kernel: None = its own choice, 0 = no chunks)
+    for portion, chunk in ((T, 0), (T, None), (T, 32), (T, 104), (150, 64), (64, 0), (5, None), (2, None)):
         state = torch.zeros(2, H, dk, dv, device="cuda")
         got = []
         for lo in range(0, T, portion):
             n = min(portion, T - lo)
             ctx = _step_context([lo], [n])
-            got.append(ops.retention(rows[lo:lo + n].contiguous(), H, dk, dv, decay, dk ** -0.5, 1e-6, state, ctx))
+            got.append(ops.retention(rows[lo:lo + n].contiguous(), H, dk, dv, decay, dk ** -0.5, 1e-6, state, ctx, chunk=chunk))
         got = torch.cat(got).double().cpu()
-        assert (got - want).abs().max() < tol, f"portion {portion}: {(got - want).abs().max()}"
+        assert (got - want).abs().max() < tol, f"portion {portion}, chunk {chunk}: {(got - want).abs().max()}"
         assert torch.count_nonzero(state[1]) == 0                 # the other slot's state is not touched
+        final = state[0].clone() if final is None else final
+        assert torch.allclose(state[0], final, rtol=1e-4, atol=1e-4), f"portion {portion}, chunk {chunk}: the state left behind differs"
+    assert ops.retention_chunk(1, 2, 300) > 0 and ops.retention_chunk(1, 2, 300) < 300      # the second case above did cut
 
 
 @gpu
