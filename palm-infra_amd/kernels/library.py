@@ -12,6 +12,8 @@ Libraries:
   ``mixers``            the mixers beside softmax attention over equal key and value sizes (retention, the selective
                         scan and its convolution, differential attention) and the stream of blocks that norm a
                         branch's output; loaded when a model has such a part
+  ``attention_diff_k<K>_v<V>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
+                        32 K and value sizes up to 16 V
 """
 from __future__ import annotations
 
@@ -41,6 +43,7 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
                 "linear_wide_gated_32.hip", "linear_wide_gated_64.hip", "linear_wide_store_128.hip", "linear_wide_gated_128.hip", "linear_mid.hip",
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
+DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
 MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
@@ -169,6 +172,9 @@ def _spec(name: str):
         return CORE_SOURCES, ()
     if name == "mixers":
         return MIXER_SOURCES, ()
+    if name.startswith("attention_diff_k"):
+        kk, vt = name[len("attention_diff_k"):].split("_v")
+        return DIFF_ATTENTION_SOURCES, (f"PALM_DIFF_KK={int(kk)}", f"PALM_DIFF_VT={int(vt)}")
     if name.startswith("attention_hd"):
         hd = int(name[len("attention_hd"):])
         return ATTENTION_SOURCES, (f"PALM_HEAD_DIM={hd}",)

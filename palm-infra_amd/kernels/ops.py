@@ -960,6 +960,50 @@ def attention_diff_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, he
     return out
 
 
+_DIFF_MFMA_SIGNATURE = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                        c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p]
+_diff_libs: dict = {}
+DIFF_MFMA_MAX_DIM, DIFF_MFMA_MAX_VDIM = 256, 256
+
+
+def diff_mfma_serves(q: torch.Tensor, dim: int, vdim: int) -> bool:
+    """The matrix-core kernel takes bfloat16, key sizes in steps of 8 and value sizes in steps of 4, up to 256."""
+    return q.dtype == BF16 and dim % 8 == 0 and vdim % 4 == 0 and dim <= DIFF_MFMA_MAX_DIM and vdim <= DIFF_MFMA_MAX_VDIM
+
+
+def attention_diff_lib(dim: int, vdim: int):
+    key = ((dim + 31) // 32, (vdim + 15) // 16)
+    if key not in _diff_libs:
+        lib = library.load(f"attention_diff_k{key[0]}_v{key[1]}")
+        lib.palm_attention_diff_mfma.argtypes, lib.palm_attention_diff_mfma.restype = _DIFF_MFMA_SIGNATURE, c_int
+        lib.palm_attention_diff_mfma_sizes.argtypes, lib.palm_attention_diff_mfma_sizes.restype = [c_int], c_int
+        if (lib.palm_attention_diff_mfma_sizes(0), lib.palm_attention_diff_mfma_sizes(1)) != (key[0] * 32, key[1] * 16):
+            raise KernelError(f"library attention_diff_k{key[0]}_v{key[1]} was built for other sizes")
+        _diff_libs[key] = lib
+    return _diff_libs[key]
+
+
+def attention_diff_mfma(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
+                        scale: float, lam: float, gain: float, eps: float) -> torch.Tensor:
+    """As ``attention_diff_exact`` for bfloat16 prompts, both products on the matrix cores."""
+    what = "attention_diff_mfma"
+    _dev(what, q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    n = q.shape[0]
+    _need(diff_mfma_serves(q, dim, vdim), f"{what}: {q.dtype}, key size {dim}, value size {vdim}")
+    _need(q.dim() == 2 and q.shape[1] == 2 * heads * dim and n == ctx.n_tokens, f"{what}: q {tuple(q.shape)} is not [n, 2*{heads}*{dim}]")
+    _check_diff_cache(what, k_cache, v_cache, block_table, kv_heads, dim, vdim)
+    _need(k_cache.dtype == BF16, f"{what}: the cache is {k_cache.dtype}, not bfloat16")
+    out = torch.empty((n, heads * vdim), dtype=BF16, device=q.device)
+    library.call(attention_diff_lib(dim, vdim), "palm_attention_diff_mfma", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
+                 heads, kv_heads, dim, vdim, float(scale), float(lam), float(gain), float(eps), _p(out))
+    return out
+
+
 def attention_diff(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps):
-    """The step's queries over the cache; picks the kernel by element type and step shape."""
+    """The step's queries over the cache; picks the kernel by element type and step shape: prompts (and portions of
+    them) in bfloat16 go to the matrix cores, single tokens and the float32 mode to the exact kernel."""
+    if not ctx.is_decode and diff_mfma_serves(q, dim, vdim):
+        return attention_diff_mfma(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps)
     return attention_diff_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps)

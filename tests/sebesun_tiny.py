@@ -41,9 +41,9 @@ CONFIGS = {
     ]},
     "Q": {"architecture": "Sebesun", "vocab": 130, "width": 48, "norm": {"eps": 2e-6}, "layers": [
         _with(_scan(40, 17, 1, 2), None),
-        _with(_att(3, 3, 24, 20, 0.25, 0.8), None),
+        _with(_att(3, 3, 24, 20, 0.1, 0.8), None),
         _with(_ret(1, 24, 80, [0.995], None), None),
-        _with(_att(2, 1, 8, 72, 0.7, 0.2), 56),
+        _with(_att(2, 1, 8, 72, 0.3, 0.2), 56),
         _with(_scan(72, 33, 9, 1), None),
     ]},
     "R": {"architecture": "Sebesun", "vocab": 97, "width": 40, "norm": {"eps": 1e-6}, "layers": [
