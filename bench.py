@@ -323,6 +323,109 @@ def other_sizes(name: str, args, sampler) -> dict:
     return out
 
 
+# ---- another design beside its closest relative -------------------------------------------------------------------
+# ``--design sebesun``: prompts and decode steps of the Sebesun presets (random weights) and of a Qwen3 model of the
+# same width, depth, head count and feed-forward width, with the time of every kernel entry point of one prompt step
+# and one decode step (launched one by one under the kernel recorder), and for the mixers' kernels the fraction of the
+# peak that binds them.
+
+def _mixer_rooflines(raw: dict, tokens: int, batch: int, context: int) -> dict:
+    """entry point -> (prefill work, prefill peak, decode work, decode peak) for one launch, by the sizes of the first
+    layer of each kind: flops against the matrix cores (attention for prompts) or the 32-bit vector units (the
+    recurrences; an exponential counts as four multiply-adds), bytes against HBM (everything in a decode step)."""
+    hbm, mfma, vec = PEAK_HBM_GBS * 1e9, PEAK_FLOPS["bf16"], PEAK_FLOPS["fp32"]
+    pairs = tokens * (tokens + 1) / 2.0
+    out = {}
+    if "layers" in raw:
+        for layer in raw["layers"]:
+            m = layer["mixer"]
+            if layer["type"] == "retention" and "palm_retention" not in out:
+                per = m["heads"] * m["dim"] * m["vdim"]
+                out["palm_retention"] = (4.0 * tokens * per, vec, 2.0 * 4 * batch * per, hbm)
+            elif layer["type"] == "mamba1" and "palm_selective_scan" not in out:
+                per = m["inner"] * m["state"]
+                out["palm_selective_scan"] = (13.0 * tokens * per, vec, 2.0 * 4 * batch * per, hbm)
+            elif layer["type"] == "attention" and "palm_attention_diff" not in out:
+                flops = 2 * 2.0 * m["heads"] * (m["dim"] + m["vdim"]) * pairs
+                kv = 2.0 * batch * context * m["kv_heads"] * (2 * m["dim"] + m["vdim"])
+                out["palm_attention_diff_mfma"] = (flops, mfma, None, None)
+                out["palm_attention_diff"] = (None, None, kv, hbm)
+    else:
+        nh, nkv, hd = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
+        out["palm_attention_prefill"] = (4.0 * nh * hd * pairs, mfma, None, None)
+        kv = 2.0 * batch * context * 2 * nkv * hd
+        out["palm_attention_decode_fused"] = out["palm_attention_decode"] = (None, None, kv, hbm)
+    return out
+
+
+def design_points(raw: dict, args, tokens: int, batch: int, context: int) -> dict:
+    """Prefill of one prompt and decode steps of ``batch`` sequences for one configuration, and its kernel table."""
+    import torch
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.kernels.profile import KernelProfile
+    from palm_infra_amd.sampling import GREEDY, DeviceSampler
+    vocab = raw["vocab"] if "vocab" in raw else raw["vocab_size"]
+    room = batch * (context + args.steps + args.warmup + 130) + tokens + 256
+    engine = Engine.from_config(raw, seed=0, dtype="bfloat16", max_tokens=room, max_seqs=batch + 2)
+    params = engine.model.weights.nbytes() / 2
+    sampler = DeviceSampler(GREEDY)
+    prefill_ms = time_prefill(engine, tokens, vocab)
+    slots = fill_contexts(engine, batch, context, vocab)
+    mean_ms, median_ms = time_decode(engine, sampler, slots, args.steps, args.warmup, vocab)
+    # every entry point of one prompt step and one decode step, launched one by one
+    rec = KernelProfile()
+    slot = engine.open()
+    with rec:
+        engine.step([StepEntry(slot, random_ids(tokens, vocab, 77), [tokens - 1])])
+        engine.step([StepEntry(s, [1], [0]) for s in slots])
+        torch.cuda.synchronize()
+    engine.close(slot)
+    roofs = _mixer_rooflines(raw, tokens, batch, context)
+    table = {}
+    for section in ("prefill", "decode"):
+        for name, calls, ms in rec.rows(section):
+            row = {"calls": calls, "us": round(ms * 1000.0 / calls, 1)}
+            work = roofs.get(name)
+            if work is not None:
+                amount, peak = (work[0], work[1]) if section == "prefill" else (work[2], work[3])
+                if amount is not None:
+                    row["frac"] = round(amount / (ms * 1e-3 / calls) / peak, 4)
+                    row["of"] = "mfma" if peak == PEAK_FLOPS["bf16"] else "fp32" if peak == PEAK_FLOPS["fp32"] else "hbm"
+            table[f"{section}:{name}"] = row
+    for s in slots:
+        engine.close(s)
+    del engine
+    torch.cuda.empty_cache()
+    return {"params_m": round(params / 1e6, 1), "prefill_tokens": tokens, "prefill_ms": round(prefill_ms, 3),
+            "prefill_tps": round(tokens * 1000.0 / prefill_ms, 1), "decode_batch": batch, "decode_context": context,
+            "decode_ms": round(mean_ms, 4), "decode_ms_median": round(median_ms, 4), "decode_tps": round(batch * 1000.0 / mean_ms, 1),
+            "kernels": table}
+
+
+def design_bench(args) -> int:
+    if args.design != "sebesun":
+        print(f"bench.py: --design {args.design}: only 'sebesun' is measured beside the default workload")
+        return 2
+    record = {"metric": "Sebesun presets beside Qwen3 models of equal width and depth: prompt and decode tok/s (bf16, random weights)",
+              "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
+              "data": "synthetic: random weights, uniform random token ids, no stop token", "sizes": {}}
+    for name in ("sebesun-2048", "sebesun-4096"):
+        raw = preset_dict(name)
+        att = next(layer["mixer"] for layer in raw["layers"] if layer["type"] == "attention")
+        ff = next(layer["mlp"]["ff"] for layer in raw["layers"] if layer["mlp"])
+        twin = dict(QWEN3_8B, hidden_size=raw["width"], num_hidden_layers=len(raw["layers"]), num_attention_heads=att["heads"],
+                    num_key_value_heads=att["kv_heads"], head_dim=raw["width"] // att["heads"],
+                    intermediate_size=(ff * 2 // 3 + 63) // 64 * 64,          # three matrices instead of two
+                    vocab_size=raw["vocab"])
+        record["sizes"][name] = {"sebesun": design_points(raw, args, PREFILL_TOKENS, BATCH, CONTEXT),
+                                 "qwen3_twin": design_points(twin, args, PREFILL_TOKENS, BATCH, CONTEXT),
+                                 "twin_config": sizes_text(twin)}
+    first = record["sizes"]["sebesun-2048"]["sebesun"]
+    record["value"], record["ms_per_step"] = first["decode_tps"], first["decode_ms"]
+    print(json.dumps(record), flush=True)
+    return 0
+
+
 def sizes_text(c) -> str:
     return (f"{c['num_hidden_layers']} layers, hidden {c['hidden_size']}, {c['num_attention_heads']} heads, "
             f"{c['num_key_value_heads']} kv heads, head_dim {c['head_dim']}, intermediate {c['intermediate_size']}, "
@@ -340,7 +443,14 @@ def main(argv=None) -> int:
     ap.add_argument("--only", default="8b,14b,32b", help="which sizes' points to measure (8b is always measured)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="tokens of the timed prompt (2,048 is the workload's; others serve profiles of longer prompts)")
+    ap.add_argument("--design", help="instead of the default workload: another design's presets beside a Qwen3 model of "
+                    "equal width and depth ('sebesun')")
     args = ap.parse_args(argv)
+    if args.design:
+        if args.gpus != 1:
+            print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not measured")
+            return 2
+        return design_bench(args)
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not measured")
         return 2

@@ -6,7 +6,8 @@
 // across), so that a lane's four results of a tile are four keys of ONE query: the softmax statistics of a query
 // then live in the lanes of its column, and the weights are already laid out as the B operand of the second product
 // O^T += V^T P^T, whose A operand reads runs of keys from the transposed value pages.  Scores leave the matrix cores
-// as 32-bit sums; maximum, exponentials, sums, the combination a1 - lambda a2 and the unit norm are 32-bit; the
+// as 32-bit sums; maximum, exponentials (base 2: the scores are scaled by scale * log2 e), sums, the combination
+// a1 - lambda a2 and the unit norm are 32-bit; the
 // weights are rounded to bfloat16 for the second product, whose sums are 32-bit again.
 //
 // Layouts as in attention_diff.hip: K [pages, 2 kv_heads, 64, dim], V [pages, kv_heads, vdim, 64].
@@ -45,7 +46,8 @@ __global__ __launch_bounds__(DM_WAVES * WAVE) void attention_diff_mfma_kernel(
     const bool live = q0 + r < n_new;
     const int start = seq_start[b];
     const int qpos = start + qi;
-    const int last_pos = start + min(q0 + 15, n_new - 1);
+    const int last_pos = start + min(q0 + 15, n_new - 1), first_pos = start + q0;
+    const float scale2 = scale * 1.4426950408889634f;
     const int kvh = h / (heads / kv_heads);
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
 
@@ -80,26 +82,37 @@ __global__ __launch_bounds__(DM_WAVES * WAVE) void attention_diff_mfma_kernel(
                 for (int kk = 0; kk < KK; ++kk) s[n] = mfma_16x16x32(load_row8(kr, kk * 32 + g * 8, dim), qf[m][kk], s[n]);
             }
             // lane (r, g) holds the keys 16 n + 4 g + i of query r
+            // scores in units of log2: a weight is then one exp2 away
             float top = -INFINITY;
+            if (pg * PAGE_TOKENS + PAGE_TOKENS - 1 > first_pos) {      // the page reaches beyond some query of the wave
 #pragma unroll
-            for (int n = 0; n < 4; ++n)
+                for (int n = 0; n < 4; ++n)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = pg * PAGE_TOKENS + 16 * n + 4 * g + i;
-                    s[n][i] = j <= qpos ? s[n][i] * scale : -INFINITY;
-                    top = fmaxf(top, s[n][i]);
-                }
+                    for (int i = 0; i < 4; ++i) {
+                        const int j = pg * PAGE_TOKENS + 16 * n + 4 * g + i;
+                        s[n][i] = j <= qpos ? s[n][i] * scale2 : -INFINITY;
+                        top = fmaxf(top, s[n][i]);
+                    }
+            } else {
+#pragma unroll
+                for (int n = 0; n < 4; ++n)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        s[n][i] *= scale2;
+                        top = fmaxf(top, s[n][i]);
+                    }
+            }
             top = fmaxf(top, __shfl_xor(top, 16, WAVE));
             top = fmaxf(top, __shfl_xor(top, 32, WAVE));
             const float m_new = fmaxf(mx[m], top);                 // finite from the first page on: key 0 is visible to all
-            const float alpha = expf(mx[m] - m_new);
+            const float alpha = exp2f(mx[m] - m_new);
             mx[m] = m_new;
             float sum = 0.f;
 #pragma unroll
             for (int n = 0; n < 4; ++n)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s[n][i] = expf(s[n][i] - m_new);
+                    s[n][i] = exp2f(s[n][i] - m_new);
                     sum += s[n][i];
                 }
             l[m] = l[m] * alpha + sum;                             // this lane's part; the groups are added at the end

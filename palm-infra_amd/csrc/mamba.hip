@@ -79,26 +79,33 @@ PALM_API int palm_causal_conv(hipStream_t stream, const void* x, int dtype, int 
 
 // ---- the scan ---------------------------------------------------------------------------------------
 // A channel's row of S is spread over a group of G lanes (G a power of two, at most 64, chosen from the state
-// size): lane j of the group holds states j, j + G, ..; a wave serves 64 / G channels, a block four waves.  For
-// every token a lane updates its states and the group adds up its part of y with shuffles.  B_t and C_t are the
-// same for all channels: a tile of tokens' rows is brought into LDS by the block.  Nothing in a token's update but
-// the multiply-add on S waits for the token before it, so the exponentials of a tile's tokens overlap.
-constexpr int SCAN_TILE = 8;
+// size): lane j of the group holds states j, j + G, ..; a block of four waves serves 256 / G channels.  The block
+// walks over a sequence's new tokens a tile at a time, in three phases with a barrier between them:
+//   in     all threads bring the tile's inputs into LDS with reads that follow the memory's rows: B_t and C_t (the
+//          same for all channels), and for the block's channels u_t and the step size softplus(dtl_t + bias),
+//          computed once for each (token, channel)
+//   scan   for every token a lane updates its states from LDS and the group adds up its part of y with shuffles;
+//          nothing but the multiply-add on S waits for the token before it, so the exponentials of a tile overlap
+//   out    all threads add the skip term, gate with silu(z_t) and store the tile's outputs row by row
+constexpr int SCAN_TILE = 16;
 constexpr int SCAN_WAVES = 4;
-constexpr int SCAN_MAX_STATE = 256;
+constexpr int SCAN_THREADS = SCAN_WAVES * WAVE;
 
 template <typename T, int G, int PER>
-__global__ __launch_bounds__(SCAN_WAVES * WAVE) void selective_scan_kernel(
+__global__ __launch_bounds__(SCAN_THREADS) void selective_scan_kernel(
     const T* __restrict__ u, const T* __restrict__ z, int z_stride, const T* __restrict__ bc, int bc_stride, int b_off, int c_off,
     const float* __restrict__ dtl, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
     const float* __restrict__ d_skip, float* __restrict__ state, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_new, const int* __restrict__ cu_new, int channels, int n_state, T* __restrict__ out) {
-    __shared__ float b_s[SCAN_TILE][SCAN_MAX_STATE], c_s[SCAN_TILE][SCAN_MAX_STATE];
-    constexpr int CH_PER_BLOCK = SCAN_WAVES * WAVE / G;
-    const int j = threadIdx.x % G;
-    const int c = blockIdx.x * CH_PER_BLOCK + threadIdx.x / G, b = blockIdx.y;
+    constexpr int CH = SCAN_THREADS / G;               // channels of a block
+    constexpr int NP = G * PER;                        // the state size, padded
+    __shared__ float b_s[SCAN_TILE][NP], c_s[SCAN_TILE][NP];
+    __shared__ float dt_s[SCAN_TILE][CH], u_s[SCAN_TILE][CH], y_s[SCAN_TILE][CH];
+    const int j = threadIdx.x % G, ch = threadIdx.x / G;
+    const int c0 = blockIdx.x * CH, b = blockIdx.y;
+    const int c = c0 + ch;
     const bool mine = c < channels;
-    const int cc = mine ? c : 0;
+    const int cc = mine ? c : channels - 1;
     const int n_new = seq_new[b];
     const size_t row0 = (size_t)cu_new[b];
     float* sp = state + ((size_t)seq_slot[b] * channels + cc) * n_state;
@@ -109,38 +116,46 @@ __global__ __launch_bounds__(SCAN_WAVES * WAVE) void selective_scan_kernel(
         S[k] = n < n_state ? sp[n] : 0.f;
         A[k] = n < n_state ? -expf(a_log[(size_t)cc * n_state + n]) : 0.f;
     }
-    const float bias = dt_bias[cc], skip = d_skip[cc];
     for (int t0 = 0; t0 < n_new; t0 += SCAN_TILE) {
         const int tt = min(SCAN_TILE, n_new - t0);
-        for (int idx = threadIdx.x; idx < tt * n_state; idx += SCAN_WAVES * WAVE) {
-            const int ti = idx / n_state, n = idx % n_state;
+        for (int idx = threadIdx.x; idx < tt * NP; idx += SCAN_THREADS) {
+            const int ti = idx / NP, n = idx % NP;
             const T* r = bc + (row0 + t0 + ti) * bc_stride;
-            b_s[ti][n] = to_float(r[b_off + n]);
-            c_s[ti][n] = to_float(r[c_off + n]);
+            b_s[ti][n] = n < n_state ? to_float(r[b_off + n]) : 0.f;
+            c_s[ti][n] = n < n_state ? to_float(r[c_off + n]) : 0.f;
+        }
+        for (int idx = threadIdx.x; idx < tt * CH; idx += SCAN_THREADS) {
+            const int ti = idx / CH, k = idx % CH;
+            const int ck = min(c0 + k, channels - 1);
+            const size_t row = row0 + t0 + ti;
+            dt_s[ti][k] = softplus_dt(dtl[row * channels + ck] + dt_bias[ck]);
+            u_s[ti][k] = to_float(u[row * channels + ck]);
         }
         __syncthreads();
 #pragma unroll
         for (int ti = 0; ti < SCAN_TILE; ++ti) {
             if (ti < tt) {
-                const size_t row = row0 + t0 + ti;
-                const float dt = softplus_dt(dtl[row * channels + cc] + bias);
-                const float uv = to_float(u[row * channels + cc]);
-                const float du = dt * uv;
+                const float dt = dt_s[ti][ch];
+                const float du = dt * u_s[ti][ch];
                 float y = 0.f;
 #pragma unroll
                 for (int k = 0; k < PER; ++k) {
                     const int n = j + k * G;
-                    if (n < n_state) {
-                        S[k] = fmaf(expf(dt * A[k]), S[k], du * b_s[ti][n]);
-                        y = fmaf(S[k], c_s[ti][n], y);
-                    }
+                    S[k] = fmaf(expf(dt * A[k]), S[k], du * b_s[ti][n]);        // beyond the state size A, B and C are zero
+                    y = fmaf(S[k], c_s[ti][n], y);
                 }
 #pragma unroll
                 for (int off = G / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);
-                if (mine && j == 0) {
-                    y = fmaf(skip, uv, y);
-                    out[row * channels + c] = from_float<T>(y * silu_f(to_float(z[row * z_stride + c])));
-                }
+                if (j == 0) y_s[ti][ch] = y;
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < tt * CH; idx += SCAN_THREADS) {
+            const int ti = idx / CH, k = idx % CH;
+            if (c0 + k < channels) {
+                const size_t row = row0 + t0 + ti;
+                const float y = fmaf(d_skip[c0 + k], u_s[ti][k], y_s[ti][k]);
+                out[row * channels + c0 + k] = from_float<T>(y * silu_f(to_float(z[row * z_stride + c0 + k])));
             }
         }
         __syncthreads();
@@ -159,13 +174,13 @@ PALM_API int palm_selective_scan(hipStream_t stream, const void* u, const void* 
                                  const float* d_skip, float* state, const int* seq_slot, const int* seq_new, const int* cu_new,
                                  int n_seqs, int channels, int n_state, void* out) {
     PALM_CHECK(n_seqs >= 0 && channels > 0 && n_state > 0, "selective_scan: seqs=%d channels=%d state=%d", n_seqs, channels, n_state);
-    PALM_CHECK(n_state <= SCAN_MAX_STATE, "selective_scan: a state of %d per channel exceeds %d", n_state, SCAN_MAX_STATE);
+    PALM_CHECK(n_state <= 256, "selective_scan: a state of %d per channel exceeds 256", n_state);
     PALM_CHECK(n_seqs <= 65535, "selective_scan: %d sequences are more than one launch takes", n_seqs);
     if (n_seqs == 0) return 0;
 #define SCAN_CASE(G, PER) { \
-        const int per_block = SCAN_WAVES * WAVE / G; \
+        const int per_block = SCAN_THREADS / G; \
         dim3 grid((channels + per_block - 1) / per_block, n_seqs); \
-        selective_scan_kernel<T, G, PER><<<grid, SCAN_WAVES * WAVE, 0, stream>>>((const T*)u, (const T*)z, z_stride, \
+        selective_scan_kernel<T, G, PER><<<grid, SCAN_THREADS, 0, stream>>>((const T*)u, (const T*)z, z_stride, \
             (const T*)bc, bc_stride, b_off, c_off, dtl, dt_bias, a_log, d_skip, state, seq_slot, seq_new, cu_new, channels, n_state, (T*)out); }
     PALM_DTYPE_SWITCH(dtype, T, {
         if (n_state <= 4) SCAN_CASE(4, 1)

@@ -7,11 +7,13 @@
 // q and k are rotated first (pairs (i, i + rot/2) of the first `rot` dimensions, cos/sin rows of the tokens'
 // positions) and k is multiplied by k_scale after the rotation; rotated values, state and sums are 32-bit.
 //
-// One block per (head, sequence), one thread per value dimension v: the thread keeps column v of S in
-// registers and walks over the sequence's new tokens, a tile of them at a time: the block rotates the tile's
-// q and k into LDS, every thread then does its column's updates and dot products for the tile's tokens, and the
-// per-token sums of squares over v are reduced for the whole tile at once.  A prompt and a single token run
-// the same code, so a prompt leaves the state that its tokens one by one leave.
+// A first pass rotates q and k of all the step's tokens into 32-bit rows.  Then one block per (head, sequence), one
+// thread per value dimension v: the thread keeps column v of S in registers and walks over the sequence's new
+// tokens.  A token's rotated q and k are the same for every thread of the block, so they are read with addresses
+// that do not depend on the thread (they come through the scalar cache and enter the multiply-adds as scalar
+// operands: no LDS, no barrier in the recurrence); the per-token sums of squares over v are reduced a tile of
+// tokens at a time.  A prompt and a single token run the same code, so a prompt leaves the state that its tokens
+// one by one leave.
 //
 // A long run of new tokens would keep only (heads x sequences) blocks busy, one after the other token.  Such a run is
 // cut into chunks of `chunk` tokens, and the recurrence's linearity does the rest in three launches:
@@ -25,14 +27,40 @@ constexpr int RET_TILE = 8;
 
 enum RetentionMode : int { RET_WHOLE = 0, RET_LOCAL = 1, RET_FROM_STARTS = 2 };
 
+// q and k of every token and head, rotated (k also scaled), 32-bit: qk[row][head][0 = q, 1 = k][dim].
+template <typename T>
+__global__ void retention_rotate_kernel(const T* __restrict__ qkvg, int row_stride, int q_off, int k_off,
+                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, float k_scale,
+                                        int n_tokens, int heads, int dim, float* __restrict__ qk) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)n_tokens * heads * dim) return;
+    const int d = (int)(idx % dim), h = (int)((idx / dim) % heads);
+    const size_t row = (size_t)(idx / ((long long)dim * heads));
+    const int half = rot / 2;
+    const T* qr = qkvg + row * row_stride + q_off + h * dim;
+    const T* kr = qkvg + row * row_stride + k_off + h * dim;
+    float qv = to_float(qr[d]), kv = to_float(kr[d]);
+    if (d < rot) {
+        const int i = d < half ? d : d - half;
+        const float c = cos_t[row * half + i], sn = sin_t[row * half + i];
+        const int partner = d < half ? d + half : d - half;
+        const float qp = to_float(qr[partner]), kp = to_float(kr[partner]);
+        // the pair (u, w) becomes (u c - w s, w c + u s)
+        qv = d < half ? qv * c - qp * sn : qv * c + qp * sn;
+        kv = d < half ? kv * c - kp * sn : kv * c + kp * sn;
+    }
+    float* o = qk + ((row * heads + h) * 2) * dim + d;
+    o[0] = qv;
+    o[dim] = kv * k_scale;
+}
+
 template <typename T, int DMAX>
-__global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, const T* __restrict__ qkvg, int row_stride, int q_off, int k_off, int v_off, int g_off,
-                                 const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
-                                 const float* __restrict__ decay, float k_scale, float eps,
+__global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, const T* __restrict__ qkvg,
+                                 int row_stride, int v_off, int g_off, const float* __restrict__ qk,
+                                 const float* __restrict__ decay, float eps,
                                  float* __restrict__ state, const int* __restrict__ seq_slot,
                                  const int* __restrict__ seq_new, const int* __restrict__ cu_new,
                                  int heads, int dim, int vdim, T* __restrict__ out) {
-    __shared__ float q_s[RET_TILE][DMAX], k_s[RET_TILE][DMAX];
     __shared__ float red[RET_TILE][16];
     const int h = blockIdx.x, b = blockIdx.y / max_chunks, c = blockIdx.y % max_chunks;
     const int v = threadIdx.x;
@@ -44,7 +72,6 @@ __global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __r
     const int row0 = cu_new[b] + (mode == RET_WHOLE ? 0 : c * chunk);
     const bool mine = v < vdim;
     const float g = decay[h];
-    const int half = rot / 2;
     float* sp = mode == RET_WHOLE ? state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + v
                                   : starts + ((((size_t)b * max_chunks + c) * heads + h) * dim) * vdim + v;
 
@@ -54,25 +81,6 @@ __global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __r
 
     for (int t0 = 0; t0 < n_new; t0 += RET_TILE) {
         const int tt = min(RET_TILE, n_new - t0);
-        for (int idx = threadIdx.x; idx < tt * dim; idx += blockDim.x) {
-            const int ti = idx / dim, d = idx % dim;
-            const size_t row = (size_t)(row0 + t0 + ti);
-            const T* qr = qkvg + row * row_stride + q_off + h * dim;
-            const T* kr = qkvg + row * row_stride + k_off + h * dim;
-            float qv = to_float(qr[d]), kv = to_float(kr[d]);
-            if (d < rot) {
-                const int i = d < half ? d : d - half;
-                const float c = cos_t[row * half + i], s = sin_t[row * half + i];
-                const int partner = d < half ? d + half : d - half;
-                const float qp = to_float(qr[partner]), kp = to_float(kr[partner]);
-                // the pair (u, w) becomes (u c - w s, w c + u s)
-                qv = d < half ? qv * c - qp * s : qv * c + qp * s;
-                kv = d < half ? kv * c - kp * s : kv * c + kp * s;
-            }
-            q_s[ti][d] = qv;
-            k_s[ti][d] = kv * k_scale;
-        }
-        __syncthreads();
         float o[RET_TILE];
 #pragma unroll
         for (int ti = 0; ti < RET_TILE; ++ti) {
@@ -80,12 +88,14 @@ __global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __r
             if (ti < tt) {
                 const size_t row = (size_t)(row0 + t0 + ti);
                 const float vv = mine ? to_float(qkvg[row * row_stride + v_off + h * vdim + v]) : 0.f;
+                const float* __restrict__ qr = qk + ((row * heads + h) * 2) * dim;       // the same for all threads
+                const float* __restrict__ kr = qr + dim;
                 float acc = 0.f;
 #pragma unroll
                 for (int d = 0; d < DMAX; ++d) {
                     if (d < dim) {
-                        S[d] = fmaf(g, S[d], k_s[ti][d] * vv);
-                        acc = fmaf(S[d], q_s[ti][d], acc);
+                        S[d] = fmaf(g, S[d], kr[d] * vv);
+                        acc = fmaf(S[d], qr[d], acc);
                     }
                 }
                 o[ti] = acc;
@@ -95,10 +105,11 @@ __global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __r
                 if (lane == 0) red[ti][wave] = ss;
             }
         }
+        if (mode == RET_LOCAL) continue;
         __syncthreads();
 #pragma unroll
         for (int ti = 0; ti < RET_TILE; ++ti) {
-            if (ti < tt && mine && mode != RET_LOCAL) {
+            if (ti < tt && mine) {
                 float total = 0.f;
                 for (int w = 0; w < n_waves; ++w) total += red[ti][w];
                 const float inv = 1.0f / sqrtf(total / (float)vdim + eps);
@@ -138,12 +149,11 @@ __global__ void retention_starts_kernel(float* __restrict__ starts, float* __res
 
 template <typename T>
 static void retention_launch(hipStream_t stream, dim3 grid, int threads, int mode, int chunk, int max_chunks, float* starts,
-                             const T* qkvg, int row_stride, int q_off, int k_off,
-                             int v_off, int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay,
-                             float k_scale, float eps, float* state, const int* seq_slot, const int* seq_new,
+                             const T* qkvg, int row_stride, int v_off, int g_off, const float* qk, const float* decay,
+                             float eps, float* state, const int* seq_slot, const int* seq_new,
                              const int* cu_new, int heads, int dim, int vdim, T* out) {
-#define RET_CASE(D) retention_kernel<T, D><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, row_stride, q_off, k_off, \
-        v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out)
+#define RET_CASE(D) retention_kernel<T, D><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, row_stride, \
+        v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out)
     if (dim <= 32) RET_CASE(32);
     else if (dim <= 64) RET_CASE(64);
     else if (dim <= 128) RET_CASE(128);
@@ -151,37 +161,41 @@ static void retention_launch(hipStream_t stream, dim3 grid, int threads, int mod
 #undef RET_CASE
 }
 
-// chunk == 0: every sequence's run in one block per head.  Else `starts` holds n_seqs * max_chunks * heads * dim * vdim
-// floats, max_chunks = ceil(max_new / chunk).
+// qk: room for n_tokens * heads * 2 * dim floats (the rotated q and k).  chunk == 0: every sequence's run in one block
+// per head.  Else `starts` holds n_seqs * max_chunks * heads * dim * vdim floats, max_chunks = ceil(max_new / chunk).
 PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int row_stride, int q_off, int k_off, int v_off,
                             int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay, float k_scale,
                             float eps, float* state, const int* seq_slot, const int* seq_new, const int* cu_new, int n_seqs,
-                            int heads, int dim, int vdim, void* out, int max_new, int chunk, float* starts) {
+                            int heads, int dim, int vdim, void* out, int max_new, int chunk, float* starts, int n_tokens,
+                            float* qk) {
     PALM_CHECK(n_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0, "retention: seqs=%d heads=%d dim=%d vdim=%d", n_seqs, heads, dim, vdim);
     PALM_CHECK(dim <= 256, "retention: a key size of %d exceeds 256", dim);
     PALM_CHECK(vdim <= 1024, "retention: a value size of %d exceeds 1024", vdim);
     PALM_CHECK(rot >= 0 && rot <= dim && rot % 2 == 0, "retention: %d rotated dimensions of %d", rot, dim);
     PALM_CHECK(rot == 0 || (cos_t && sin_t), "retention: a rotation needs its cos and sin rows");
     PALM_CHECK(chunk >= 0 && (chunk == 0 || (starts && max_new > 0)), "retention: chunks of %d tokens need their starting states", chunk);
-    if (n_seqs == 0) return 0;
+    PALM_CHECK(n_tokens >= 0 && (n_tokens == 0 || qk), "retention: the rotated q and k need their room");
+    if (n_seqs == 0 || n_tokens == 0) return 0;
     const int max_chunks = chunk > 0 ? (max_new + chunk - 1) / chunk : 1;
     PALM_CHECK(heads <= 65535 && (long long)n_seqs * max_chunks <= 65535, "retention: %d heads / %d sequences x %d chunks are more than one launch takes",
                heads, n_seqs, max_chunks);
     const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
     dim3 grid(heads, n_seqs * max_chunks);
+    const long long rot_threads = (long long)n_tokens * heads * dim;
     PALM_DTYPE_SWITCH(dtype, T, {
+        retention_rotate_kernel<T><<<(unsigned)((rot_threads + 255) / 256), 256, 0, stream>>>((const T*)qkvg, row_stride, q_off, k_off, cos_t,
+                                                                                             sin_t, rot, k_scale, n_tokens, heads, dim, qk);
         if (chunk == 0) {
-            retention_launch<T>(stream, grid, threads, RET_WHOLE, 1 << 30, 1, nullptr, (const T*)qkvg, row_stride, q_off, k_off, v_off,
-                                g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+            retention_launch<T>(stream, grid, threads, RET_WHOLE, 1 << 30, 1, nullptr, (const T*)qkvg, row_stride, v_off, g_off, qk, decay,
+                                eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
         } else {
-            retention_launch<T>(stream, grid, threads, RET_LOCAL, chunk, max_chunks, starts, (const T*)qkvg, row_stride, q_off, k_off,
-                                v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
+            retention_launch<T>(stream, grid, threads, RET_LOCAL, chunk, max_chunks, starts, (const T*)qkvg, row_stride, v_off, g_off, qk,
+                                decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
             const int elems = heads * dim * vdim;
             retention_starts_kernel<<<dim3((elems + 255) / 256, n_seqs), 256, 0, stream>>>(starts, state, decay, seq_slot, seq_new, chunk,
                                                                                          max_chunks, heads, dim * vdim);
-            retention_launch<T>(stream, grid, threads, RET_FROM_STARTS, chunk, max_chunks, starts, (const T*)qkvg, row_stride, q_off,
-                                k_off, v_off, g_off, cos_t, sin_t, rot, decay, k_scale, eps, state, seq_slot, seq_new, cu_new, heads, dim,
-                                vdim, (T*)out);
+            retention_launch<T>(stream, grid, threads, RET_FROM_STARTS, chunk, max_chunks, starts, (const T*)qkvg, row_stride, v_off, g_off,
+                                qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);
         }
     });
     PALM_LAUNCHED();

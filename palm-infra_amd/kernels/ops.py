@@ -763,7 +763,7 @@ _MIXER_SIGNATURES = {
     "palm_xielu": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_longlong],
     "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
                        c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
-                       c_void_p],
+                       c_void_p, c_int, c_void_p],
     "palm_causal_conv": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_void_p],
     "palm_selective_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -771,7 +771,8 @@ _MIXER_SIGNATURES = {
     "palm_diff_qkv_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                             c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_int],
     "palm_attention_diff": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p],
+                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p, c_int,
+                            c_void_p, c_int],
 }
 _mixers = None
 
@@ -859,6 +860,7 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
             _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"retention: rotation rows are float32 [{n}, {rot // 2}]")
     out = torch.empty((n, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
     chunk = retention_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
+    rotated = torch.empty((n, heads, 2, dim), dtype=F32, device=qkvg.device)          # q and k after the rotation, 32-bit
     starts = None
     if chunk:
         max_chunks = -(-ctx.max_new // chunk)
@@ -866,7 +868,7 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
     library.call(mixers(), "palm_retention", _stream(), _p(qkvg), _code(qkvg, "retention"), qkvg.shape[1], 0, heads * dim,
                  2 * heads * dim, 2 * heads * dim + heads * vdim, _p(cos), _p(sin), int(rot), _p(decay), float(k_scale), float(eps),
                  _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, dim, vdim, _p(out),
-                 int(ctx.max_new), chunk, _p(starts))
+                 int(ctx.max_new), chunk, _p(starts), n, _p(rotated))
     return out
 
 
@@ -942,10 +944,21 @@ def diff_qkv_store(qkv: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim:
     return q
 
 
+DIFF_BLOCKS_WANTED = 1024         # a decode step's key ranges are cut into slices until about this many blocks run
+
+
+def diff_slices(ctx, heads: int) -> int:
+    """Into how many slices the exact kernel cuts every key range: only a decode step's (few queries, long ranges)."""
+    if not ctx.is_decode:
+        return 1
+    pages = max(1, (ctx.max_total + PAGE_TOKENS - 1) // PAGE_TOKENS)
+    return max(1, min(pages, DIFF_BLOCKS_WANTED // max(1, ctx.n_seqs * heads), 64))
+
+
 def attention_diff_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, heads: int, kv_heads: int, dim: int, vdim: int,
-                         scale: float, lam: float, gain: float, eps: float) -> torch.Tensor:
+                         scale: float, lam: float, gain: float, eps: float, n_slices: int | None = None) -> torch.Tensor:
     """Differential attention of the step's queries over the cache in 32-bit arithmetic: out [n, heads * vdim] =
-    unit_rms(a1 - lam * a2) * gain per head."""
+    unit_rms(a1 - lam * a2) * gain per head.  ``n_slices``: see ``diff_slices`` (None: chosen here)."""
     what = "attention_diff"
     _dev(what, q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
     _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
@@ -954,9 +967,12 @@ def attention_diff_exact(q: torch.Tensor, k_cache, v_cache, block_table, ctx, he
     _check_diff_cache(what, k_cache, v_cache, block_table, kv_heads, dim, vdim)
     _need(k_cache.dtype == q.dtype, f"{what}: cache is {k_cache.dtype}, queries are {q.dtype}")
     out = torch.empty((n, heads * vdim), dtype=q.dtype, device=q.device)
+    n_slices = diff_slices(ctx, heads) if n_slices is None else int(n_slices)
+    _need(n_slices == 1 or ctx.is_decode, f"{what}: only a decode step's key ranges are cut into slices")
+    work = torch.empty((n * heads * n_slices * 2 * (vdim + 2),), dtype=F32, device=q.device) if n_slices > 1 else None
     library.call(mixers(), "palm_attention_diff", _stream(), _p(q), _code(q, what), _p(k_cache), _p(v_cache), _p(block_table),
                  block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
-                 heads, kv_heads, dim, vdim, float(scale), float(lam), float(gain), float(eps), _p(out))
+                 heads, kv_heads, dim, vdim, float(scale), float(lam), float(gain), float(eps), _p(out), n_slices, _p(work), n)
     return out
 
 

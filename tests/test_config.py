@@ -128,10 +128,11 @@ def test_run_order_is_data_and_is_checked():
 
 def test_named_sizes_are_data_and_load():
     from palm_infra_amd.config import ConfigError, config_source, preset_dict, preset_names
-    assert {"tiny-a", "tiny-b", "qwen3-8b", "qwen3-14b", "qwen3-32b"} <= set(preset_names())
+    assert {"tiny-a", "tiny-b", "qwen3-8b", "qwen3-14b", "qwen3-32b", "tiny-sebesun", "sebesun-2048", "sebesun-4096"} <= set(preset_names())
     for name in preset_names():
         cfg = config_from_dict(preset_dict(name))
-        assert cfg.spec().vocab_size == preset_dict(name)["vocab_size"]
+        raw = preset_dict(name)
+        assert cfg.spec().vocab_size == (raw["vocab_size"] if "vocab_size" in raw else raw["vocab"])
     assert config_source("tiny-b")["head_dim"] == 32
     with pytest.raises(ConfigError, match="unknown size 'qwen9'.*tiny-a"):
         config_source("qwen9")
