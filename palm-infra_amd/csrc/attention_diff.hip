@@ -174,8 +174,8 @@ __global__ __launch_bounds__(DIFF_WAVES * WAVE) void attention_diff_kernel(
             for (int e = 0; e < N; ++e) { p0[e] = __shfl(p[0], j0 + e, WAVE); p1[e] = __shfl(p[1], j0 + e, WAVE); }
 #pragma unroll
             for (int i = 0; i < DIFF_ACC; ++i) {
-                const int d = lane + i * WAVE;
-                if (d < vdim) {
+                if (i * WAVE < vdim) {                        // the same for all lanes; a lane beyond vdim reads the last row
+                    const int d = min(lane + i * WAVE, vdim - 1);
                     float v[N];
                     Pieces<T>::load(vp + (size_t)d * PAGE_TOKENS + j0, v);
 #pragma unroll

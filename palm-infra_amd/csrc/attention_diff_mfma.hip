@@ -27,8 +27,10 @@ constexpr int DM_QUERIES = 16 * DM_WAVES;
 PALM_API int palm_attention_diff_mfma_sizes(int which) { return which == 0 ? KK * 32 : VT * 16; }
 
 __device__ inline bf16x8 load_row8(const bf16_t* row, int col, int dim) {
-    // eight values of a row from column `col`; columns beyond `dim` are zero (dim is a multiple of eight)
-    return col < dim ? load_bf16x8(row + col) : zero_bf16x8();
+    // eight values of a row from column `col`; columns beyond `dim` are zero (dim is a multiple of eight).  The read
+    // itself is unconditional (of the row's last eight values where the column lies beyond it): no branch around it
+    const bf16x8 v = load_bf16x8(row + min(col, dim - 8));
+    return col < dim ? v : zero_bf16x8();
 }
 
 __global__ __launch_bounds__(DM_WAVES * WAVE) void attention_diff_mfma_kernel(
@@ -136,15 +138,10 @@ __global__ __launch_bounds__(DM_WAVES * WAVE) void attention_diff_mfma_kernel(
             const bf16_t* vr = vp + (size_t)min(vd, vdim - 1) * PAGE_TOKENS;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                bf16x8 vf;
-                if (vd < vdim) {
-                    const uint2 lo = *reinterpret_cast<const uint2*>(vr + 32 * half + 4 * g);
-                    const uint2 hi = *reinterpret_cast<const uint2*>(vr + 32 * half + 16 + 4 * g);
-                    const uint4 both = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                    vf = __builtin_bit_cast(bf16x8, both);
-                } else {
-                    vf = zero_bf16x8();
-                }
+                const uint2 lo = *reinterpret_cast<const uint2*>(vr + 32 * half + 4 * g);       // row min(vd, vdim - 1): always there
+                const uint2 hi = *reinterpret_cast<const uint2*>(vr + 32 * half + 16 + 4 * g);
+                const uint4 both = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                const bf16x8 vf = vd < vdim ? __builtin_bit_cast(bf16x8, both) : zero_bf16x8();
                 acc[0][vt] = mfma_16x16x32(vf, pf[0][half], acc[0][vt]);
                 acc[1][vt] = mfma_16x16x32(vf, pf[1][half], acc[1][vt]);
             }

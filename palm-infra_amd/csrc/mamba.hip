@@ -88,6 +88,23 @@ PALM_API int palm_causal_conv(hipStream_t stream, const void* x, int dtype, int 
 //          nothing but the multiply-add on S waits for the token before it, so the exponentials of a tile overlap
 //   out    all threads add the skip term, gate with silu(z_t) and store the tile's outputs row by row
 constexpr int SCAN_TILE = 16;
+
+// Sum over groups of G consecutive lanes (G a power of two), every lane gets its group's sum.  Within a row of 16
+// lanes the partners come through the data-parallel lane crossbar of the vector unit (one instruction a step: quads
+// swap, halves of 8 and rows of 16 mirror: any pairing of disjoint partial sums does); only steps across rows go
+// through the permute unit.
+template <int CTRL> __device__ inline float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int G> __device__ inline float group_sum(float y) {
+    if constexpr (G >= 2) y += dpp_move<0xB1>(y);            // quad_perm [1, 0, 3, 2]
+    if constexpr (G >= 4) y += dpp_move<0x4E>(y);            // quad_perm [2, 3, 0, 1]
+    if constexpr (G >= 8) y += dpp_move<0x141>(y);           // row_half_mirror
+    if constexpr (G >= 16) y += dpp_move<0x140>(y);          // row_mirror
+    if constexpr (G >= 32) y += __shfl_xor(y, 16, WAVE);
+    if constexpr (G >= 64) y += __shfl_xor(y, 32, WAVE);
+    return y;
+}
 constexpr int SCAN_WAVES = 4;
 constexpr int SCAN_THREADS = SCAN_WAVES * WAVE;
 
@@ -132,23 +149,26 @@ __global__ __launch_bounds__(SCAN_THREADS) void selective_scan_kernel(
             u_s[ti][k] = to_float(u[row * channels + ck]);
         }
         __syncthreads();
+#define SCAN_TOKEN(ti) { \
+            const float dt = dt_s[ti][ch]; \
+            const float du = dt * u_s[ti][ch]; \
+            float y = 0.f; \
+            _Pragma("unroll") for (int k = 0; k < PER; ++k) { \
+                const int n = j + k * G; \
+                S[k] = fmaf(expf(dt * A[k]), S[k], du * b_s[ti][n]);        /* beyond the state size A, B and C are zero */ \
+                y = fmaf(S[k], c_s[ti][n], y); \
+            } \
+            y = group_sum<G>(y); \
+            if (j == 0) y_s[ti][ch] = y; }
+        if (tt == SCAN_TILE) {                                  // a whole tile: no test between its tokens
 #pragma unroll
-        for (int ti = 0; ti < SCAN_TILE; ++ti) {
-            if (ti < tt) {
-                const float dt = dt_s[ti][ch];
-                const float du = dt * u_s[ti][ch];
-                float y = 0.f;
+            for (int ti = 0; ti < SCAN_TILE; ++ti) SCAN_TOKEN(ti)
+        } else {
 #pragma unroll
-                for (int k = 0; k < PER; ++k) {
-                    const int n = j + k * G;
-                    S[k] = fmaf(expf(dt * A[k]), S[k], du * b_s[ti][n]);        // beyond the state size A, B and C are zero
-                    y = fmaf(S[k], c_s[ti][n], y);
-                }
-#pragma unroll
-                for (int off = G / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);
-                if (j == 0) y_s[ti][ch] = y;
-            }
+            for (int ti = 0; ti < SCAN_TILE; ++ti)
+                if (ti < tt) SCAN_TOKEN(ti)
         }
+#undef SCAN_TOKEN
         __syncthreads();
         for (int idx = threadIdx.x; idx < tt * CH; idx += SCAN_THREADS) {
             const int ti = idx / CH, k = idx % CH;

@@ -9,10 +9,9 @@
 //
 // A first pass rotates q and k of all the step's tokens into 32-bit rows.  Then one block per (head, sequence), one
 // thread per value dimension v: the thread keeps column v of S in registers and walks over the sequence's new
-// tokens.  A token's rotated q and k are the same for every thread of the block, so they are read with addresses
-// that do not depend on the thread (they come through the scalar cache and enter the multiply-adds as scalar
-// operands: no LDS, no barrier in the recurrence); the per-token sums of squares over v are reduced a tile of
-// tokens at a time.  A prompt and a single token run the same code, so a prompt leaves the state that its tokens
+// tokens.  A token's rotated q and k are the same for every thread of the block: each wave reads the two rows once,
+// one value a lane, and broadcasts value d to all its lanes as a scalar operand of the multiply-adds (no LDS and no
+// barrier in the recurrence); the per-token sums of squares over v are reduced a tile of tokens at a time.  A prompt and a single token run the same code, so a prompt leaves the state that its tokens
 // one by one leave.
 //
 // A long run of new tokens would keep only (heads x sequences) blocks busy, one after the other token.  Such a run is
@@ -27,15 +26,19 @@ constexpr int RET_TILE = 8;
 
 enum RetentionMode : int { RET_WHOLE = 0, RET_LOCAL = 1, RET_FROM_STARTS = 2 };
 
-// q and k of every token and head, rotated (k also scaled), 32-bit: qk[row][head][0 = q, 1 = k][dim].
+// q and k of every token and head, rotated (k also scaled), 32-bit: qk[row][head][0 = q, 1 = k][pad], pad >= dim the
+// key size that the main kernel is compiled for; the columns beyond dim are zero, so that the main kernel's loops
+// over pad need no test (a zero k leaves its row of S zero, a zero q adds nothing).
 template <typename T>
 __global__ void retention_rotate_kernel(const T* __restrict__ qkvg, int row_stride, int q_off, int k_off,
                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, float k_scale,
-                                        int n_tokens, int heads, int dim, float* __restrict__ qk) {
+                                        int n_tokens, int heads, int dim, int pad, float* __restrict__ qk) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (long long)n_tokens * heads * dim) return;
-    const int d = (int)(idx % dim), h = (int)((idx / dim) % heads);
-    const size_t row = (size_t)(idx / ((long long)dim * heads));
+    if (idx >= (long long)n_tokens * heads * pad) return;
+    const int d = (int)(idx % pad), h = (int)((idx / pad) % heads);
+    const size_t row = (size_t)(idx / ((long long)pad * heads));
+    float* o = qk + ((row * heads + h) * 2) * pad + d;
+    if (d >= dim) { o[0] = 0.f; o[pad] = 0.f; return; }
     const int half = rot / 2;
     const T* qr = qkvg + row * row_stride + q_off + h * dim;
     const T* kr = qkvg + row * row_stride + k_off + h * dim;
@@ -49,19 +52,22 @@ __global__ void retention_rotate_kernel(const T* __restrict__ qkvg, int row_stri
         qv = d < half ? qv * c - qp * sn : qv * c + qp * sn;
         kv = d < half ? kv * c - kp * sn : kv * c + kp * sn;
     }
-    float* o = qk + ((row * heads + h) * 2) * dim + d;
     o[0] = qv;
-    o[dim] = kv * k_scale;
+    o[pad] = kv * k_scale;
 }
 
-template <typename T, int DMAX>
-__global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, const T* __restrict__ qkvg,
+// MAXT: the most threads of a block (the value size, rounded up to whole waves): what the compiler may assume when it
+// hands out registers.  A thread keeps DMAX values of S; up to 256 threads a block they all stay in registers.
+template <typename T, int DMAX, int MAXT>
+__global__ __launch_bounds__(MAXT) void retention_kernel(int mode, int chunk, int max_chunks, float* __restrict__ starts, const T* __restrict__ qkvg,
                                  int row_stride, int v_off, int g_off, const float* __restrict__ qk,
                                  const float* __restrict__ decay, float eps,
                                  float* __restrict__ state, const int* __restrict__ seq_slot,
                                  const int* __restrict__ seq_new, const int* __restrict__ cu_new,
                                  int heads, int dim, int vdim, T* __restrict__ out) {
     __shared__ float red[RET_TILE][16];
+    __shared__ float o_s[RET_TILE][MAXT];
+    constexpr int QREGS = (DMAX + WAVE - 1) / WAVE;
     const int h = blockIdx.x, b = blockIdx.y / max_chunks, c = blockIdx.y % max_chunks;
     const int v = threadIdx.x;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
@@ -75,48 +81,67 @@ __global__ void retention_kernel(int mode, int chunk, int max_chunks, float* __r
     float* sp = mode == RET_WHOLE ? state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + v
                                   : starts + ((((size_t)b * max_chunks + c) * heads + h) * dim) * vdim + v;
 
+    // the reads are unconditional (of a row and a column that exist) and what does not belong is set to zero after:
+    // no branch between them, so that they are all under way at once
     float S[DMAX];
+    {
+        const float* at = sp - v + min(v, vdim - 1);
+        const bool zero = mode == RET_LOCAL || !mine;
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) S[d] = (mine && d < dim && mode != RET_LOCAL) ? sp[(size_t)d * vdim] : 0.f;
+        for (int d = 0; d < DMAX; ++d) {
+            const float s0 = at[(size_t)min(d, dim - 1) * vdim];
+            S[d] = (zero || d >= dim) ? 0.f : s0;
+        }
+    }
 
+    // A token's inputs: the thread's value, and of the token's q and k rows (the same for all threads) one value a
+    // lane, which the wave hands to all its lanes as scalars.  The next token's are read while this one's are used.
+    const int vc = min(v, vdim - 1);
+    auto read_token = [&](int t, float& vv, float (&qv)[QREGS], float (&kv)[QREGS]) {
+        const size_t row = (size_t)(row0 + t);
+        vv = to_float(qkvg[row * row_stride + v_off + h * vdim + vc]);
+        const float* __restrict__ qr = qk + ((row * heads + h) * 2) * DMAX;
+#pragma unroll
+        for (int c = 0; c < QREGS; ++c) {
+            const int at = min(c * WAVE + lane, DMAX - 1);             // (a key size of 32: the upper lanes repeat)
+            qv[c] = qr[at];
+            kv[c] = qr[DMAX + at];
+        }
+    };
+    float vv, qv[QREGS], kv[QREGS];
+    if (n_new > 0) read_token(0, vv, qv, kv);
     for (int t0 = 0; t0 < n_new; t0 += RET_TILE) {
         const int tt = min(RET_TILE, n_new - t0);
-        float o[RET_TILE];
+        for (int ti = 0; ti < tt; ++ti) {                        // not unrolled: the body is DMAX steps long already
+            float vn, qn[QREGS], kn[QREGS];
+            read_token(min(t0 + ti + 1, n_new - 1), vn, qn, kn);
+            if (!mine) vv = 0.f;
+            float acc = 0.f;
 #pragma unroll
-        for (int ti = 0; ti < RET_TILE; ++ti) {
-            o[ti] = 0.f;
-            if (ti < tt) {
-                const size_t row = (size_t)(row0 + t0 + ti);
-                const float vv = mine ? to_float(qkvg[row * row_stride + v_off + h * vdim + v]) : 0.f;
-                const float* __restrict__ qr = qk + ((row * heads + h) * 2) * dim;       // the same for all threads
-                const float* __restrict__ kr = qr + dim;
-                float acc = 0.f;
-#pragma unroll
-                for (int d = 0; d < DMAX; ++d) {
-                    if (d < dim) {
-                        S[d] = fmaf(g, S[d], kr[d] * vv);
-                        acc = fmaf(S[d], qr[d], acc);
-                    }
-                }
-                o[ti] = acc;
+            for (int d = 0; d < DMAX; ++d) {
+                const float qd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, qv[d / WAVE]), d % WAVE));
+                const float kd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kv[d / WAVE]), d % WAVE));
+                S[d] = fmaf(g, S[d], kd * vv);
+                acc = fmaf(S[d], qd, acc);
             }
             if (mode != RET_LOCAL) {
-                const float ss = wave_sum(o[ti] * o[ti]);
+                o_s[ti][v] = acc;
+                const float ss = wave_sum(acc * acc);
                 if (lane == 0) red[ti][wave] = ss;
             }
+            vv = vn;
+#pragma unroll
+            for (int c = 0; c < QREGS; ++c) { qv[c] = qn[c]; kv[c] = kn[c]; }
         }
         if (mode == RET_LOCAL) continue;
         __syncthreads();
-#pragma unroll
-        for (int ti = 0; ti < RET_TILE; ++ti) {
-            if (ti < tt && mine) {
-                float total = 0.f;
-                for (int w = 0; w < n_waves; ++w) total += red[ti][w];
-                const float inv = 1.0f / sqrtf(total / (float)vdim + eps);
-                const size_t row = (size_t)(row0 + t0 + ti);
-                const float gate = to_float(qkvg[row * row_stride + g_off + h * vdim + v]);
-                out[row * ((size_t)heads * vdim) + h * vdim + v] = from_float<T>(o[ti] * inv * (gate / (1.0f + expf(-gate))));
-            }
+        for (int ti = 0; ti < tt; ++ti) {
+            float total = 0.f;
+            for (int w = 0; w < n_waves; ++w) total += red[ti][w];
+            const float inv = 1.0f / sqrtf(total / (float)vdim + eps);
+            const size_t row = (size_t)(row0 + t0 + ti);
+            const float gate = to_float(qkvg[row * row_stride + g_off + h * vdim + vc]);
+            if (mine) out[row * ((size_t)heads * vdim) + h * vdim + v] = from_float<T>(o_s[ti][v] * inv * (gate / (1.0f + expf(-gate))));
         }
         __syncthreads();
     }
@@ -152,17 +177,21 @@ static void retention_launch(hipStream_t stream, dim3 grid, int threads, int mod
                              const T* qkvg, int row_stride, int v_off, int g_off, const float* qk, const float* decay,
                              float eps, float* state, const int* seq_slot, const int* seq_new,
                              const int* cu_new, int heads, int dim, int vdim, T* out) {
-#define RET_CASE(D) retention_kernel<T, D><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, row_stride, \
-        v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out)
-    if (dim <= 32) RET_CASE(32);
-    else if (dim <= 64) RET_CASE(64);
-    else if (dim <= 128) RET_CASE(128);
-    else RET_CASE(256);
+#define RET_CASE(D) { if (threads <= 256) retention_kernel<T, D, 256><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, \
+            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out); \
+        else retention_kernel<T, D, 1024><<<grid, threads, 0, stream>>>(mode, chunk, max_chunks, starts, qkvg, \
+            row_stride, v_off, g_off, qk, decay, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, out); }
+    if (dim <= 32) RET_CASE(32)
+    else if (dim <= 64) RET_CASE(64)
+    else if (dim <= 128) RET_CASE(128)
+    else RET_CASE(256)
 #undef RET_CASE
 }
 
-// qk: room for n_tokens * heads * 2 * dim floats (the rotated q and k).  chunk == 0: every sequence's run in one block
+// qk: room for n_tokens * heads * 2 * pad floats (the rotated q and k; pad = palm_retention_pad(dim)).  chunk == 0: every sequence's run in one block
 // per head.  Else `starts` holds n_seqs * max_chunks * heads * dim * vdim floats, max_chunks = ceil(max_new / chunk).
+PALM_API int palm_retention_pad(int dim) { return dim <= 32 ? 32 : dim <= 64 ? 64 : dim <= 128 ? 128 : 256; }
+
 PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int row_stride, int q_off, int k_off, int v_off,
                             int g_off, const float* cos_t, const float* sin_t, int rot, const float* decay, float k_scale,
                             float eps, float* state, const int* seq_slot, const int* seq_new, const int* cu_new, int n_seqs,
@@ -181,10 +210,11 @@ PALM_API int palm_retention(hipStream_t stream, const void* qkvg, int dtype, int
                heads, n_seqs, max_chunks);
     const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
     dim3 grid(heads, n_seqs * max_chunks);
-    const long long rot_threads = (long long)n_tokens * heads * dim;
+    const int pad = palm_retention_pad(dim);
+    const long long rot_threads = (long long)n_tokens * heads * pad;
     PALM_DTYPE_SWITCH(dtype, T, {
         retention_rotate_kernel<T><<<(unsigned)((rot_threads + 255) / 256), 256, 0, stream>>>((const T*)qkvg, row_stride, q_off, k_off, cos_t,
-                                                                                             sin_t, rot, k_scale, n_tokens, heads, dim, qk);
+                                                                                             sin_t, rot, k_scale, n_tokens, heads, dim, pad, qk);
         if (chunk == 0) {
             retention_launch<T>(stream, grid, threads, RET_WHOLE, 1 << 30, 1, nullptr, (const T*)qkvg, row_stride, v_off, g_off, qk, decay,
                                 eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out);

@@ -764,6 +764,7 @@ _MIXER_SIGNATURES = {
     "palm_retention": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
                        c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
                        c_void_p, c_int, c_void_p],
+    "palm_retention_pad": [c_int],
     "palm_causal_conv": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_void_p],
     "palm_selective_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -860,7 +861,8 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
             _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot // 2), f"retention: rotation rows are float32 [{n}, {rot // 2}]")
     out = torch.empty((n, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
     chunk = retention_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
-    rotated = torch.empty((n, heads, 2, dim), dtype=F32, device=qkvg.device)          # q and k after the rotation, 32-bit
+    # q and k after the rotation, 32-bit, in rows padded to the key size that the kernel is compiled for
+    rotated = torch.empty((n, heads, 2, mixers().palm_retention_pad(dim)), dtype=F32, device=qkvg.device)
     starts = None
     if chunk:
         max_chunks = -(-ctx.max_new // chunk)
