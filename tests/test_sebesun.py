@@ -192,10 +192,11 @@ def test_one_layer_of_one_kind(tmp_path_factory, kind, dtype):
 
 
 @gpu
-def test_stream_kernel_norms_adds_and_averages_over_depth():
+@pytest.mark.parametrize("W", [50, 64, 2048, 5000, 20000])      # no multiple of four, narrow, wide, several groups a thread, beyond them
+def test_stream_kernel_norms_adds_and_averages_over_depth(W):
     from palm_infra_amd.kernels import ops
     torch.manual_seed(1)
-    n, W, J = 7, 50, 3
+    n, J = 7, 3
     x = torch.randn(n, W, device="cuda")
     y = torch.randn(n, W, device="cuda") * 3
     w = torch.rand(W, device="cuda") + 0.5
