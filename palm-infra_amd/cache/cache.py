@@ -226,13 +226,18 @@ class ModelCache:
     entry's cache: ``shares[i]`` is that entry's index)."""
 
     def __init__(self, needs: list[list], shares: list[int | None], max_tokens: int, max_seqs: int | None,
-                 max_positions: int | None, dtype: torch.dtype, device):
+                 max_positions: int | None, dtype: torch.dtype, device, page_slack: int = 0):
+        """``page_slack``: pages beyond those of ``max_tokens``, for a caller whose ``max_tokens`` counts the tokens that
+        live sequences hold and not the part of each one's last page that stays empty: one page for each sequence that may
+        be live at once.  The longest sequence stays what ``max_tokens`` allows."""
         if max_tokens <= 0:
             raise ValueError(f"max_tokens = {max_tokens} must be positive")
+        if page_slack < 0:
+            raise ValueError(f"page_slack = {page_slack} must not be negative")
         self.device, self.dtype = device, dtype
-        n_pages = pages_for(max_tokens)
+        self.max_tokens = pages_for(max_tokens) * PAGE_TOKENS
+        n_pages = pages_for(max_tokens) + int(page_slack)
         self.max_seqs = int(max_seqs) if max_seqs else min(n_pages, 1024)
-        self.max_tokens = n_pages * PAGE_TOKENS
         self.max_seq_tokens = min(max_positions, self.max_tokens) if max_positions else self.max_tokens
         max_pages_per_slot = pages_for(self.max_seq_tokens)
         self.pad_slot = self.max_seqs

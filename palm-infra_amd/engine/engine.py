@@ -60,7 +60,7 @@ class Engine:
     takes_fed = True             # step(entries, fed=..) takes tokens that are still on the device
 
     def __init__(self, config, spec, weights, dtype: torch.dtype, max_tokens: int, max_seqs: int | None = None,
-                 device="cuda:0", graphs: bool = True, max_step_tokens: int = 32768):
+                 device="cuda:0", graphs: bool = True, max_step_tokens: int = 32768, page_slack: int = 0):
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError(f"the engine runs on a GPU; device {device!r} was asked for and there is no CPU path")
@@ -70,7 +70,7 @@ class Engine:
         self.config, self.spec, self.dtype = config, spec, dtype
         self.model = DecoderModel(spec, weights, dtype, self.device)
         needs, shares = self.model.cache_plan()
-        self.cache = ModelCache(needs, shares, max_tokens, max_seqs, spec.max_positions, dtype, self.device)
+        self.cache = ModelCache(needs, shares, max_tokens, max_seqs, spec.max_positions, dtype, self.device, page_slack=page_slack)
         self.vocab_size = spec.vocab_size
         self.graphs_enabled = bool(graphs)
         self._decode_graphs: dict = {}            # (batch bucket, length bucket) -> recorded step, least recently used first

@@ -21,6 +21,11 @@ import sys
 from pathlib import Path
 
 
+# ``--max-tokens`` counts the tokens that live requests hold, not the rest of each one's last page: the cache gets a page
+# more for each of this many requests that may be live at once
+LIVE_REQUESTS = 256
+
+
 def replay(engine, lines, out_dir, report=print) -> None:
     out_dir = Path(out_dir)
     out_dir.mkdir(parents=True, exist_ok=True)
@@ -60,16 +65,18 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="the most tokens that live requests hold at any time (each rounded up to 64)")
+                    help="the most tokens that live requests hold at any time (the cache also has a page of 64 for each of "
+                    f"up to {LIVE_REQUESTS} live requests, for the part of a request's last page that stays empty)")
     args = ap.parse_args(argv)
     from ..cache import CacheFull
     from .engine import Engine
     try:
         if args.random:
             from ..config import config_source
-            engine = Engine.from_config(config_source(args.random), seed=args.seed, dtype=args.dtype, max_tokens=args.max_tokens)
+            engine = Engine.from_config(config_source(args.random), seed=args.seed, dtype=args.dtype, max_tokens=args.max_tokens,
+                                        page_slack=LIVE_REQUESTS)
         else:
-            engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+            engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens, page_slack=LIVE_REQUESTS)
     except (ValueError, FileNotFoundError, RuntimeError) as e:
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr)
         return 1

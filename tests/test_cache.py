@@ -242,3 +242,32 @@ def test_a_need_of_a_kind_the_cache_has_never_heard_of():
     assert c.nbytes() >= sum(g.nbytes() for g in mine)
     c.reserve([(s, 100)]); c.commit([(s, 100)])
     c.check()
+
+
+def test_page_slack_holds_many_short_sequences_but_no_longer_ones():
+    """A caller that counts the tokens live sequences hold (not the empty rest of each one's last page) asks for a page
+    more for each sequence that may be live; the longest sequence stays what max_tokens allows."""
+    need = KVNeed(2, 8)
+    tight = ModelCache([[need]], [None], 128, None, None, torch.float32, "cpu")
+    slack = ModelCache([[need]], [None], 128, None, None, torch.float32, "cpu", page_slack=6)
+    assert tight.max_seqs == 2 and slack.max_seqs == 8 and slack.max_seq_tokens == tight.max_seq_tokens == 128
+    slots = [slack.open() for _ in range(8)]
+    slack.reserve([(s, 16) for s in slots])              # 128 tokens in eight sequences: eight pages
+    slack.commit([(s, 16) for s in slots])
+    slack.check()
+    with pytest.raises(CacheFull):
+        slack.reserve([(slots[0], 113)])                 # 16 + 113 tokens are more than one sequence may hold
+    a = tight.open()
+    b = tight.open()
+    tight.reserve([(a, 16), (b, 16)])
+    with pytest.raises(CacheFull):
+        tight.open()
+
+
+def test_keys_and_values_of_different_head_counts_and_sizes_share_a_group():
+    need = KVNeed(4, 24, None, value_heads=2, value_dim=40)
+    cache = ModelCache([[need], [need]], [None, None], 256, None, None, torch.float32, "cpu")
+    group = cache.groups_of(KVNeed)[0]
+    assert group.k.shape == (2, 5, 4, PAGE_TOKENS, 24) and group.v.shape == (2, 5, 2, 40, PAGE_TOKENS)
+    assert group.nbytes() == (group.k.numel() + group.v.numel()) * 4
+    assert cache.layer_caches[1].k.shape == (5, 4, PAGE_TOKENS, 24) and cache.layer_caches[1].v.shape == (5, 2, 40, PAGE_TOKENS)

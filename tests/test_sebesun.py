@@ -514,3 +514,30 @@ def test_command_line_generates_for_the_design(tmp_path_factory, capsys):
                     "--dtype", "float32", "--ignore-eos"])
     assert rc == 0
     assert " ".join(str(t) for t in P.greedy(cfg, w, [5, 6, 7], 6)) in capsys.readouterr().out
+
+
+@gpu
+def test_trace_replay_of_many_short_requests_counted_by_their_tokens(tmp_path_factory, tmp_path):
+    """bin/trace_run as a child process: six requests of 70 tokens in one batch and then one token each, with
+    --max-tokens counting the tokens they hold (426) and not the pages they touch (twelve)."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    d = model_dir(tmp_path_factory, "P", "float32")
+    reqs = S.prompts(raw_of("P"), [71] * 6, seed=11)
+    steps = [{"step": 0, "entries": [{"id": f"r{i}", "tokens": r[:70], "want": [0, 69]} for i, r in enumerate(reqs)], "end": []},
+             {"step": 1, "entries": [{"id": f"r{i}", "tokens": r[70:], "want": [0]} for i, r in enumerate(reqs)], "end": [f"r{i}" for i in range(6)]}]
+    root = Path(__file__).resolve().parent.parent
+    proc = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32", "--out", str(tmp_path / "o"),
+                           "--max-tokens", "426"], input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [line for line in proc.stdout.splitlines() if line.startswith("done")] == ["done 0", "done 1"]
+    V = raw_of("P")["vocab"]
+    first = torch.from_numpy(np.fromfile(tmp_path / "o" / "0.f32", dtype="<f4").reshape(-1, V).copy())
+    second = torch.from_numpy(np.fromfile(tmp_path / "o" / "1.f32", dtype="<f4").reshape(-1, V).copy())
+    for i, r in enumerate(reqs):
+        ref = reference(tmp_path_factory, "P", "float32", r)
+        assert_close(first[2 * i:2 * i + 2], ref[[0, 69]], "float32", f"request {i}, prompt")
+        assert_close(second[i:i + 1], ref[70:71], "float32", f"request {i}, decoded")
