@@ -12,8 +12,8 @@ Libraries:
   ``mixers``            the mixers beside softmax attention over equal key and value sizes (retention, the selective
                         scan and its convolution, differential attention) and the stream of blocks that norm a
                         branch's output; loaded when a model has such a part
-  ``attention_diff_k<K>_v<V>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
-                        32 K and value sizes up to 16 V
+  ``attention_diff_k<K>_v<V>_q<Q>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
+                        32 K, value sizes up to 16 V and Q tiles of 16 queries a wave
 """
 from __future__ import annotations
 
@@ -173,8 +173,9 @@ def _spec(name: str):
     if name == "mixers":
         return MIXER_SOURCES, ()
     if name.startswith("attention_diff_k"):
-        kk, vt = name[len("attention_diff_k"):].split("_v")
-        return DIFF_ATTENTION_SOURCES, (f"PALM_DIFF_KK={int(kk)}", f"PALM_DIFF_VT={int(vt)}")
+        kk, rest = name[len("attention_diff_k"):].split("_v")
+        vt, qt = rest.split("_q")
+        return DIFF_ATTENTION_SOURCES, (f"PALM_DIFF_KK={int(kk)}", f"PALM_DIFF_VT={int(vt)}", f"PALM_DIFF_QT={int(qt)}")
     if name.startswith("attention_hd"):
         hd = int(name[len("attention_hd"):])
         return ATTENTION_SOURCES, (f"PALM_HEAD_DIM={hd}",)

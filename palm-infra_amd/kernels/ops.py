@@ -989,14 +989,24 @@ def diff_mfma_serves(q: torch.Tensor, dim: int, vdim: int) -> bool:
     return q.dtype == BF16 and dim % 8 == 0 and vdim % 4 == 0 and dim <= DIFF_MFMA_MAX_DIM and vdim <= DIFF_MFMA_MAX_VDIM
 
 
+def diff_query_tiles(vdim: int) -> int:
+    """Tiles of 16 queries a wave of the matrix-core kernel: two where the output tiles of both maps then still fit a
+    lane's registers."""
+    import os
+    forced = os.environ.get("PALM_DIFF_QUERY_TILES")
+    if forced:
+        return int(forced)
+    return 2 if (vdim + 15) // 16 <= 8 else 1
+
+
 def attention_diff_lib(dim: int, vdim: int):
-    key = ((dim + 31) // 32, (vdim + 15) // 16)
+    key = ((dim + 31) // 32, (vdim + 15) // 16, diff_query_tiles(vdim))
     if key not in _diff_libs:
-        lib = library.load(f"attention_diff_k{key[0]}_v{key[1]}")
+        lib = library.load(f"attention_diff_k{key[0]}_v{key[1]}_q{key[2]}")
         lib.palm_attention_diff_mfma.argtypes, lib.palm_attention_diff_mfma.restype = _DIFF_MFMA_SIGNATURE, c_int
         lib.palm_attention_diff_mfma_sizes.argtypes, lib.palm_attention_diff_mfma_sizes.restype = [c_int], c_int
-        if (lib.palm_attention_diff_mfma_sizes(0), lib.palm_attention_diff_mfma_sizes(1)) != (key[0] * 32, key[1] * 16):
-            raise KernelError(f"library attention_diff_k{key[0]}_v{key[1]} was built for other sizes")
+        if tuple(lib.palm_attention_diff_mfma_sizes(i) for i in range(3)) != (key[0] * 32, key[1] * 16, key[2]):
+            raise KernelError(f"library attention_diff_k{key[0]}_v{key[1]}_q{key[2]} was built for other sizes")
         _diff_libs[key] = lib
     return _diff_libs[key]
 

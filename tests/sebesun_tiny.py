@@ -47,7 +47,7 @@ CONFIGS = {
         _with(_scan(72, 33, 9, 1), None),
     ]},
     "R": {"architecture": "Sebesun", "vocab": 97, "width": 40, "norm": {"eps": 1e-6}, "layers": [
-        _with(_ret(2, 32, 64, [0.999, 0.98], {"dims": 32, "base": 1000000.0}), 64),
+        _with(_ret(2, 32, 48, [0.999, 0.98], {"dims": 32, "base": 250000.0}), 64),
     ]},
 }
 SEEDS = {"P": 11, "Q": 12, "R": 13}

@@ -73,7 +73,7 @@ def test_random_model_folder_is_read_by_the_plain_implementation(tmp_path):
     from palm_infra_amd.weights import write_random_model
     d = write_random_model(S.CONFIGS["R"], 5, tmp_path / "m", "bfloat16")
     cfg, w = P.read_model(d)
-    assert cfg["layers"][0]["type"] == "retention" and w["l0.mix.q"].shape == (64, 40)
+    assert cfg["layers"][0]["type"] == "retention" and w["l0.mix.q"].shape == (64, 40) and w["l0.mix.v"].shape == (96, 40)
     logits = P.forward(cfg, w, [1, 2, 3])
     assert logits.shape == (3, 97) and torch.isfinite(logits).all()
 
