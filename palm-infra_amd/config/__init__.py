@@ -4,8 +4,9 @@ from .registry import (ConfigError, config_class_for, config_from_dict, config_f
 from .spec import LayerCall, ModelSpec, PartSpec, Stored, TensorRef, joined, tensor
 from .qwen3 import Qwen3Config
 from .sebesun import SebesunConfig
+from .pazilorn import PazilornConfig
 
 __all__ = ["ConfigError", "config_class_for", "config_from_dict", "config_from_dir", "config_source", "preset_dict",
            "preset_names", "register_architecture",
            "registered_architectures", "LayerCall", "ModelSpec", "PartSpec", "Stored", "TensorRef", "joined", "tensor",
-           "Qwen3Config", "SebesunConfig"]
+           "Qwen3Config", "SebesunConfig", "PazilornConfig"]

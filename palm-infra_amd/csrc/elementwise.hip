@@ -11,10 +11,11 @@ PALM_DEFINE_LAST_ERROR()
 PALM_API int palm_page_tokens() { return PAGE_TOKENS; }
 
 // ---- embedding ------------------------------------------------------------------------------------
-// One block per token.  An id outside the table gives a row of NaN: visible, and no read out of bounds.
+// One block per token: the table's row times `scale` (1 for a plain table).  An id outside the table gives a row of
+// NaN: visible, and no read out of bounds.
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
-                             int hidden, int vocab) {
+                             int hidden, int vocab, float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     float* dst = out + (size_t)t * hidden;
@@ -23,15 +24,15 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
         return;
     }
     const TW* src = table + (size_t)id * hidden;
-    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(src[d]);
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(src[d]) * scale;     // (times 1 is exact)
 }
 
 PALM_API int palm_embed(hipStream_t stream, const void* table, int table_dtype, const int* ids, int n_tokens,
-                        int hidden, int vocab, float* out) {
+                        int hidden, int vocab, float* out, float scale) {
     PALM_CHECK(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed: n_tokens=%d hidden=%d vocab=%d", n_tokens, hidden, vocab);
     if (n_tokens == 0) return 0;
     PALM_DTYPE_SWITCH(table_dtype, TW,
-        embed_kernel<TW><<<n_tokens, 256, 0, stream>>>((const TW*)table, ids, out, hidden, vocab));
+        embed_kernel<TW><<<n_tokens, 256, 0, stream>>>((const TW*)table, ids, out, hidden, vocab, scale));
     PALM_LAUNCHED();
     return 0;
 }

@@ -25,7 +25,7 @@ __global__ void causal_conv_kernel(const T* __restrict__ x, int x_stride, const 
     if (c >= channels || ti >= seq_new[b]) return;
     const size_t row0 = (size_t)cu_new[b];
     const float* st = conv_state + (size_t)seq_slot[b] * (taps - 1) * channels;      // [taps-1, channels], oldest first
-    float acc = bias[c];
+    float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int at = ti - (taps - 1) + j;                 // index among the step's tokens; negative: from the state
         const float v = at >= 0 ? to_float(x[(row0 + at) * x_stride + c]) : st[(size_t)(taps - 1 + at) * channels + c];

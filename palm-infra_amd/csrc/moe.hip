@@ -1,0 +1,173 @@
+// A feed-forward of routed experts: every token goes through `top` of `experts` small gated feed-forwards.
+//
+//   route      from a token's router logits (32-bit): the `top` largest (the lower index wins a tie), and as their
+//              weights the softmax over those logits alone
+//   few rows (a decode step): nothing is planned on the host, every (token, choice) reads its expert's weights itself
+//     expert_gate_up   mid[t, c, f] = silu(G_e h_t)[f] * (U_e h_t)[f],  e = chosen[t, c]           (32-bit)
+//     expert_down      out[t, :] = sum_c weight[t, c] * D_e mid[t, c, :]  in the order of c        (32-bit)
+//   many rows (a prompt): the host groups the (token, choice) pairs by expert, the products are the library's
+//     gather_rows      xs[p, :] = h[src[p], :]
+//     scatter_add      out[rows[i], :] += weight[i] * y[i, :]      (an expert's rows are distinct tokens: no two
+//                      threads meet, and the experts are added one after the other)
+#include "common.h"
+
+constexpr int ROUTE_MAX_PER_LANE = 8;            // up to 512 experts
+
+// One wave per token.
+__global__ __launch_bounds__(WAVE) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
+                                                         int* __restrict__ chosen, float* __restrict__ weight) {
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x;
+    float z[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+        const int e = i * WAVE + lane;
+        z[i] = e < experts ? logits[t * experts + e] : -INFINITY;
+    }
+    float first = 0.f, sum = 0.f, mine = 0.f;
+    for (int c = 0; c < top; ++c) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+            const int e = i * WAVE + lane;
+            if (e < experts && (z[i] > best || (z[i] == best && e < at))) { best = z[i]; at = e; }
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, WAVE);
+            const int oa = __shfl_xor(at, off, WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        if (c == 0) first = best;
+        const float p = expf(best - first);                  // the first is the largest
+        sum += p;
+        if (lane == c) mine = p;                             // lane c keeps choice c's weight
+        if (lane == 0) chosen[t * top + c] = at;
+#pragma unroll
+        for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i)
+            if (i * WAVE + lane == at) z[i] = -INFINITY;
+    }
+    if (lane < top) weight[t * top + lane] = mine / sum;
+}
+
+// grid (blocks of rows of the expert's inner size, top, tokens); a wave computes a gate row and its up row at a time.
+constexpr int MOE_THREADS = 256;
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(MOE_THREADS) void expert_gate_up_kernel(const T* __restrict__ h, const TW* __restrict__ gate_up,
+                                                                     const int* __restrict__ chosen, int top, int width, int ff,
+                                                                     int rows_per_block, float* __restrict__ mid) {
+    extern __shared__ float h_s[];                  // [width]
+    const int t = blockIdx.z, c = blockIdx.y;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = MOE_THREADS / WAVE;
+    for (int d = threadIdx.x; d < width; d += MOE_THREADS) h_s[d] = to_float(h[(size_t)t * width + d]);
+    __syncthreads();
+    const int e = chosen[(size_t)t * top + c];
+    const TW* w = gate_up + (size_t)e * 2 * ff * width;
+    const int f_end = min(ff, (int)(blockIdx.x + 1) * rows_per_block);
+    for (int f = blockIdx.x * rows_per_block + wave; f < f_end; f += n_waves) {
+        const TW* gr = w + (size_t)f * width;
+        const TW* ur = w + (size_t)(ff + f) * width;
+        float g = 0.f, u = 0.f;
+        for (int d = lane; d < width; d += WAVE) {
+            const float hv = h_s[d];
+            g = fmaf(to_float(gr[d]), hv, g);
+            u = fmaf(to_float(ur[d]), hv, u);
+        }
+        g = wave_sum(g);
+        u = wave_sum(u);
+        if (lane == 0) mid[((size_t)t * top + c) * ff + f] = g / (1.0f + expf(-g)) * u;
+    }
+}
+
+// grid (blocks of output rows, tokens); a wave computes one output value at a time, the choices one after the other.
+template <typename TW>
+__global__ __launch_bounds__(MOE_THREADS) void expert_down_kernel(const float* __restrict__ mid, const TW* __restrict__ down,
+                                                                  const int* __restrict__ chosen, const float* __restrict__ weight,
+                                                                  int top, int width, int ff, int rows_per_block,
+                                                                  float* __restrict__ out) {
+    extern __shared__ float m_s[];                  // [top][ff]
+    const int t = blockIdx.y;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = MOE_THREADS / WAVE;
+    for (int i = threadIdx.x; i < top * ff; i += MOE_THREADS) m_s[i] = mid[(size_t)t * top * ff + i];
+    __syncthreads();
+    const int r_end = min(width, (int)(blockIdx.x + 1) * rows_per_block);
+    for (int r = blockIdx.x * rows_per_block + wave; r < r_end; r += n_waves) {
+        float total = 0.f;
+        for (int c = 0; c < top; ++c) {
+            const TW* wr = down + ((size_t)chosen[(size_t)t * top + c] * width + r) * ff;
+            float acc = 0.f;
+            for (int f = lane; f < ff; f += WAVE) acc = fmaf(to_float(wr[f]), m_s[c * ff + f], acc);
+            total = fmaf(weight[(size_t)t * top + c], wave_sum(acc), total);
+        }
+        if (lane == 0) out[(size_t)t * width + r] = total;
+    }
+}
+
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ h, const int* __restrict__ src, int width, T* __restrict__ xs) {
+    const size_t p = blockIdx.x;
+    const T* from = h + (size_t)src[p] * width;
+    for (int d = threadIdx.x; d < width; d += blockDim.x) xs[p * width + d] = from[d];
+}
+
+template <typename T>
+__global__ void scatter_add_kernel(const T* __restrict__ y, const int* __restrict__ rows, const float* __restrict__ weight,
+                                   int width, float* __restrict__ out) {
+    const size_t i = blockIdx.x;
+    float* to = out + (size_t)rows[i] * width;
+    const float w = weight[i];
+    for (int d = threadIdx.x; d < width; d += blockDim.x) to[d] = fmaf(w, to_float(y[i * width + d]), to[d]);
+}
+
+PALM_API int palm_moe_route(hipStream_t stream, const float* logits, int n_tokens, int experts, int top, int* chosen, float* weight) {
+    PALM_CHECK(n_tokens >= 0 && experts > 0 && top > 0 && top <= experts, "moe_route: n=%d experts=%d top=%d", n_tokens, experts, top);
+    PALM_CHECK(experts <= ROUTE_MAX_PER_LANE * WAVE, "moe_route: %d experts exceed %d", experts, ROUTE_MAX_PER_LANE * WAVE);
+    PALM_CHECK(top <= WAVE, "moe_route: %d choices a token exceed %d", top, WAVE);
+    if (n_tokens == 0) return 0;
+    moe_route_kernel<<<n_tokens, WAVE, 0, stream>>>(logits, experts, top, chosen, weight);
+    PALM_LAUNCHED();
+    return 0;
+}
+
+// h [n, width]; gate_up [experts, 2 ff, width] (an expert's gate rows, then its up rows); down [experts, width, ff];
+// chosen, weight [n, top]; mid: room for n * top * ff floats; out float32 [n, width].
+PALM_API int palm_moe_experts(hipStream_t stream, const void* h, int dtype, const void* gate_up, const void* down, int w_dtype,
+                              const int* chosen, const float* weight, int n_tokens, int top, int width, int ff, float* mid,
+                              float* out) {
+    PALM_CHECK(n_tokens >= 0 && top > 0 && width > 0 && ff > 0, "moe_experts: n=%d top=%d width=%d ff=%d", n_tokens, top, width, ff);
+    PALM_CHECK(width <= 16384 && (long long)top * ff <= 16384, "moe_experts: width %d / top x ff %d x %d exceed what a block holds", width, top, ff);
+    PALM_CHECK(n_tokens <= 65535 && top <= 65535, "moe_experts: %d tokens x %d choices are more than one launch takes", n_tokens, top);
+    if (n_tokens == 0) return 0;
+    // blocks enough to fill the chip, but no fewer than four rows a wave
+    const int up_rows = max(16, (ff + 15) / 16), up_blocks = (ff + up_rows - 1) / up_rows;
+    const int down_rows = max(16, (width + 63) / 64), down_blocks = (width + down_rows - 1) / down_rows;
+    PALM_DTYPE_SWITCH(dtype, T, {
+        PALM_DTYPE_SWITCH(w_dtype, TW, {
+            expert_gate_up_kernel<T, TW><<<dim3(up_blocks, top, n_tokens), MOE_THREADS, width * sizeof(float), stream>>>(
+                (const T*)h, (const TW*)gate_up, chosen, top, width, ff, up_rows, mid);
+            expert_down_kernel<TW><<<dim3(down_blocks, n_tokens), MOE_THREADS, (size_t)top * ff * sizeof(float), stream>>>(
+                mid, (const TW*)down, chosen, weight, top, width, ff, down_rows, out);
+        });
+    });
+    PALM_LAUNCHED();
+    return 0;
+}
+
+PALM_API int palm_gather_rows(hipStream_t stream, const void* h, int dtype, const int* src, int n_rows, int width, void* xs) {
+    PALM_CHECK(n_rows >= 0 && width > 0, "gather_rows: rows=%d width=%d", n_rows, width);
+    if (n_rows == 0) return 0;
+    PALM_DTYPE_SWITCH(dtype, T, gather_rows_kernel<T><<<n_rows, 256, 0, stream>>>((const T*)h, src, width, (T*)xs));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+PALM_API int palm_scatter_add(hipStream_t stream, const void* y, int dtype, const int* rows, const float* weight, int n_rows,
+                              int width, float* out) {
+    PALM_CHECK(n_rows >= 0 && width > 0, "scatter_add: rows=%d width=%d", n_rows, width);
+    if (n_rows == 0) return 0;
+    PALM_DTYPE_SWITCH(dtype, T, scatter_add_kernel<T><<<n_rows, 256, 0, stream>>>((const T*)y, rows, weight, width, out));
+    PALM_LAUNCHED();
+    return 0;
+}

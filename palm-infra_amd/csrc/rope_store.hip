@@ -412,25 +412,27 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
 }
 
 // cos/sin rows [n_tokens, half] for the step's positions: angle = position * inv_freq[i], in 32-bit,
-// with the full-range sin and cos (engine/input_prep.cpp:17-30).
+// with the full-range sin and cos (engine/input_prep.cpp:17-30); both times `magnitude` (1 for a plain rotation;
+// a rotation with stretched frequencies lengthens the rotated vectors by a factor of its own).
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                  float* __restrict__ cos_t, float* __restrict__ sin_t, int n_tokens, int half) {
+                                  float* __restrict__ cos_t, float* __restrict__ sin_t, int n_tokens, int half,
+                                  float magnitude) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n_tokens * half) return;
     const float ang = (float)positions[i / half] * inv_freq[i % half];
     float s, c;
     sincosf(ang, &s, &c);
-    cos_t[i] = c;
-    sin_t[i] = s;
+    cos_t[i] = c * magnitude;
+    sin_t[i] = s * magnitude;
 }
 
 PALM_API int palm_rope_table(hipStream_t stream, const int* positions, const float* inv_freq, float* cos_t,
-                             float* sin_t, int n_tokens, int half) {
+                             float* sin_t, int n_tokens, int half, float magnitude) {
     PALM_CHECK(n_tokens >= 0 && half > 0, "rope_table: tokens=%d half=%d", n_tokens, half);
     if (n_tokens == 0) return 0;
     const long long total = (long long)n_tokens * half;
     PALM_CHECK(total < (1ll << 31), "rope_table: %lld entries are more than one launch takes", total);
-    rope_table_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(positions, inv_freq, cos_t, sin_t, n_tokens, half);
+    rope_table_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(positions, inv_freq, cos_t, sin_t, n_tokens, half, magnitude);
     PALM_LAUNCHED();
     return 0;
 }

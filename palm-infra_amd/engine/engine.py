@@ -95,6 +95,8 @@ class Engine:
         model_dir = Path(model_dir)
         config = config_from_dir(model_dir)
         files = ModelFiles(model_dir)
+        if hasattr(config, "with_tensor_shapes"):       # an architecture some of whose sizes only the tensors' shapes give
+            config = config.with_tensor_shapes({name: files.shape(name) for name in files.names()})
         spec = config.spec(files.names())
         weights = load_weights(spec, files, dt, device, strict=strict_weights)
         return cls(config, spec, weights, dt, max_tokens or 16384, device=device, **options)

@@ -10,8 +10,9 @@ Libraries:
   ``core``              every kernel that does not depend on the head size
   ``attention_hd<N>``   the matrix-core attention kernels, compiled for one head size
   ``mixers``            the mixers beside softmax attention over equal key and value sizes (retention, the selective
-                        scan and its convolution, differential attention) and the stream of blocks that norm a
-                        branch's output; loaded when a model has such a part
+                        scan and its convolution, differential attention, the delta rule, attention over compressed
+                        rows), routed experts, and the stream of blocks that norm a branch's output; loaded when a
+                        model has such a part
   ``attention_diff_k<K>_v<V>_q<Q>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
                         32 K, value sizes up to 16 V and Q tiles of 16 queries a wave
 """
@@ -44,7 +45,8 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
 DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
-MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip"]
+MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
+                 "latent_attention.hip", "moe.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
 

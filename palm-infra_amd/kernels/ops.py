@@ -19,7 +19,7 @@ _CODES = {F32: 0, BF16: 1}
 PAGE_TOKENS = 64
 
 _SIGNATURES = {
-    "palm_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "palm_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_float],
     "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
                      c_void_p, c_int, c_int, c_longlong],
     "palm_swiglu": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
@@ -30,7 +30,7 @@ _SIGNATURES = {
     "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_float],
-    "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
+    "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float],
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -111,8 +111,8 @@ def _i32(what: str, *tensors) -> None:
 
 # ---- elementwise ----------------------------------------------------------------------------------
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :] as float32."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] * scale as float32."""
     _dev("embed", table, ids, out)
     _i32("embed", ids)
     _need(table.dim() == 2 and ids.dim() == 1, f"embed: table {tuple(table.shape)}, ids {tuple(ids.shape)}")
@@ -121,7 +121,8 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
     if out is None:
         out = torch.empty((n, hidden), dtype=F32, device=table.device)
     _need(out.shape == (n, hidden) and out.dtype == F32, f"embed: out {tuple(out.shape)} {out.dtype}")
-    library.call(core(), "palm_embed", _stream(), _p(table), _code(table, "embed table"), _p(ids), n, hidden, vocab, _p(out))
+    library.call(core(), "palm_embed", _stream(), _p(table), _code(table, "embed table"), _p(ids), n, hidden, vocab, _p(out),
+                 float(scale))
     return out
 
 
@@ -271,15 +272,15 @@ def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions:
     return q_out
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
-    """cos, sin [n, half] float32 of positions[t] * inv_freq[i]."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0):
+    """cos, sin [n, half] float32 of positions[t] * inv_freq[i], both times ``magnitude``."""
     _dev("rope_table", positions, inv_freq)
     _i32("rope_table", positions)
     _need(positions.dim() == 1 and inv_freq.dim() == 1 and inv_freq.dtype == F32, "rope_table: positions [n] int32, inv_freq [half] float32")
     n, half = positions.shape[0], inv_freq.shape[0]
     cos = torch.empty((n, half), dtype=F32, device=positions.device)
     sin = torch.empty_like(cos)
-    library.call(core(), "palm_rope_table", _stream(), _p(positions), _p(inv_freq), _p(cos), _p(sin), n, half)
+    library.call(core(), "palm_rope_table", _stream(), _p(positions), _p(inv_freq), _p(cos), _p(sin), n, half, float(magnitude))
     return cos, sin
 
 
@@ -774,6 +775,24 @@ _MIXER_SIGNATURES = {
     "palm_attention_diff": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p, c_int,
                             c_void_p, c_int],
+    "palm_add_normed_scaled": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float, c_float, c_int, c_int, c_void_p, c_float,
+                               c_void_p, c_int],
+    "palm_softcap": [c_void_p, c_void_p, c_float, c_longlong],
+    "palm_delta_pad": [c_int],
+    "palm_delta_rule": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                        c_void_p, c_void_p, c_void_p, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                        c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p],
+    "palm_latent_prep": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p,
+                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int],
+    "palm_latent_query": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "palm_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                              c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "palm_latent_output": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "palm_moe_route": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+    "palm_moe_experts": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_void_p, c_void_p],
+    "palm_gather_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "palm_scatter_add": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 _mixers = None
 
@@ -874,16 +893,16 @@ def retention(qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.
     return out
 
 
-def causal_conv(xz: torch.Tensor, channels: int, weight: torch.Tensor, bias: torch.Tensor, conv_state: torch.Tensor, ctx) -> torch.Tensor:
-    """silu(bias + a causal convolution per channel) over the first ``channels`` columns of xz [n, >= channels];
+def causal_conv(xz: torch.Tensor, channels: int, weight: torch.Tensor, bias: torch.Tensor | None, conv_state: torch.Tensor, ctx) -> torch.Tensor:
+    """silu(bias + a causal convolution per channel) (``bias`` None: none) over the first ``channels`` columns of xz [n, >= channels];
     weight float32 [channels, taps] (last column: the current token), conv_state float32 [slots, taps - 1, channels]:
     each sequence's last inputs, read and left updated."""
     _dev("causal_conv", xz, weight, bias, conv_state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     _i32("causal_conv", ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     taps = weight.shape[1]
     _need(xz.dim() == 2 and xz.shape[1] >= channels and xz.shape[0] == ctx.n_tokens, f"causal_conv: input {tuple(xz.shape)}")
-    _need(weight.shape == (channels, taps) and weight.dtype == F32 and bias.shape == (channels,) and bias.dtype == F32,
-          f"causal_conv: weight {tuple(weight.shape)} {weight.dtype}, bias {tuple(bias.shape)} {bias.dtype}")
+    _need(weight.shape == (channels, taps) and weight.dtype == F32 and (bias is None or (bias.shape == (channels,) and bias.dtype == F32)),
+          f"causal_conv: weight {tuple(weight.shape)} {weight.dtype}, bias {None if bias is None else tuple(bias.shape)}")
     _need(conv_state.dim() == 3 and conv_state.shape[1:] == (max(taps - 1, 0), channels) and conv_state.dtype == F32,
           f"causal_conv: state {tuple(conv_state.shape)} is not float32 [slots, {taps - 1}, {channels}]")
     out = torch.empty((xz.shape[0], channels), dtype=xz.dtype, device=xz.device)
@@ -1036,3 +1055,201 @@ def attention_diff(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, 
     if not ctx.is_decode and diff_mfma_serves(q, dim, vdim):
         return attention_diff_mfma(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps)
     return attention_diff_exact(q, k_cache, v_cache, block_table, ctx, heads, kv_heads, dim, vdim, scale, lam, gain, eps)
+
+
+# ---- blocks that norm a branch on both sides; a cap on the logits -------------------------------------------------
+
+def add_normed_scaled(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, gain: float,
+                      next_weight: torch.Tensor | None = None, next_eps: float = 0.0, out_dtype: torch.dtype | None = None):
+    """x += gain * (delta / sqrt(mean(delta^2) + eps) * weight), row by row, in place (x float32 [n, width]).  With
+    ``next_weight``: also returns x / sqrt(mean(x^2) + next_eps) * next_weight in ``out_dtype``, made in the same pass
+    (what the norm that reads the stream next would give); else returns None."""
+    _dev("add_normed_scaled", x, delta, weight, next_weight)
+    _need(x.dim() == 2 and x.dtype == F32 and delta.shape == x.shape, f"add_normed_scaled: x {tuple(x.shape)} {x.dtype}, delta {tuple(delta.shape)}")
+    n, width = x.shape
+    for w in (weight, next_weight):
+        _need(w is None or (w.shape == (width,) and w.dtype == F32), f"add_normed_scaled: a norm's weight is float32 [{width}]")
+    out = None
+    if next_weight is not None:
+        out = torch.empty((n, width), dtype=out_dtype or F32, device=x.device)
+    library.call(mixers(), "palm_add_normed_scaled", _stream(), _p(x), _p(delta), _code(delta, "add_normed_scaled delta"), _p(weight),
+                 float(eps), float(gain), n, width, _p(next_weight), float(next_eps), _p(out),
+                 _code(out, "add_normed_scaled out") if out is not None else 0)
+    return out
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (float32).  Returns logits."""
+    _dev("softcap", logits)
+    _need(logits.dtype == F32 and cap > 0, f"softcap: float32 logits and a positive cap, not {logits.dtype} and {cap}")
+    library.call(mixers(), "palm_softcap", _stream(), _p(logits), float(cap), logits.numel())
+    return logits
+
+
+# ---- the delta rule ------------------------------------------------------------------------------------------------
+
+def delta_rule(u: torch.Tensor, offsets: tuple, b: torch.Tensor, a: torch.Tensor, gate: torch.Tensor, a_log: torch.Tensor,
+               dt_bias: torch.Tensor, norm_w: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, q_scale: float,
+               unit_eps: float, eps: float, state: torch.Tensor, ctx) -> torch.Tensor:
+    """The step's tokens through the recurrence of a gated delta rule with one decay per key channel.
+
+    u [n, >= 2 kv_heads dim + heads vdim]: the convolution's output with q, k, v at the columns ``offsets``; b [n, heads]
+    (a view of rows is fine: its row stride is passed on): the write strengths before the sigmoid; a float32 [n, heads * dim]
+    and gate float32 [n, heads * vdim] (views likewise): the decays' rows before bias and softplus, the output gate before
+    its sigmoid; state float32 [slots, heads, dim, vdim], read and left updated.  Returns [n, heads * vdim]: the heads'
+    outputs, each normed over vdim with ``norm_w`` and gated."""
+    what = "delta_rule"
+    _dev(what, u, a_log, dt_bias, norm_w, state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    _i32(what, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
+    n = u.shape[0]
+    q_off, k_off, v_off = (int(o) for o in offsets)
+    _need(u.dim() == 2 and n == ctx.n_tokens and max(q_off, k_off) + kv_heads * dim <= u.shape[1] and v_off + heads * vdim <= u.shape[1],
+          f"{what}: rows {tuple(u.shape)} do not hold q, k ({kv_heads} x {dim}) and v ({heads} x {vdim}) at {offsets}")
+    for t, cols, dt, nm in ((b, heads, u.dtype, "write strengths"), (a, heads * dim, F32, "decay rows"), (gate, heads * vdim, F32, "gate rows")):
+        _need(t.is_cuda and t.dim() == 2 and t.shape == (n, cols) and t.dtype == dt and (n == 0 or t.stride(1) == 1),
+              f"{what}: the {nm} are {dt} [{n}, {cols}] with contiguous rows, not {t.dtype} {tuple(t.shape)}")
+    _need(a_log.shape == (heads,) and a_log.dtype == F32 and dt_bias.shape == (heads * dim,) and dt_bias.dtype == F32
+          and norm_w.shape == (vdim,) and norm_w.dtype == F32, f"{what}: A_log [{heads}], dt_bias [{heads * dim}] and the norm's weight [{vdim}] are float32")
+    _need(state.dim() == 4 and state.shape[1:] == (heads, dim, vdim) and state.dtype == F32,
+          f"{what}: state {tuple(state.shape)} {state.dtype} is not float32 [slots, {heads}, {dim}, {vdim}]")
+    out = torch.empty((n, heads * vdim), dtype=u.dtype, device=u.device)
+    prep = torch.empty((n, heads, 3, mixers().palm_delta_pad(dim)), dtype=F32, device=u.device)
+    beta = torch.empty((n, heads), dtype=F32, device=u.device)
+    library.call(mixers(), "palm_delta_rule", _stream(), _p(u), _code(u, what), u.stride(0), q_off, k_off, v_off, _p(b), b.stride(0),
+                 _p(a), a.stride(0), _p(gate), gate.stride(0), _p(a_log), _p(dt_bias), _p(norm_w), float(q_scale), float(unit_eps),
+                 float(eps), _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, kv_heads, dim, vdim,
+                 _p(out), n, _p(prep), _p(beta))
+    return out
+
+
+# ---- attention over one compressed row per position -----------------------------------------------------------------
+
+def latent_prep(down: torch.Tensor, q_rank: int, kv_off: int, kv_rank: int, rot_dim: int, q_norm_w, kv_norm_w, eps: float,
+                cos, sin, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, write_cache: bool = True) -> torch.Tensor:
+    """down [n, >= kv_off + kv_rank + rot_dim]: the query latent at column 0, the key/value latent at ``kv_off`` and the key
+    part to rotate behind it.  Returns the normed query latent [n, q_rank]; writes [normed latent | rotated key part] into
+    each token's row of ``rows_cache`` [pages, PAGE_TOKENS, kv_rank + rot_dim]."""
+    what = "latent_prep"
+    _dev(what, down, q_norm_w, kv_norm_w, cos, sin, rows_cache, block_table, ctx.positions, ctx.tok_slot)
+    _i32(what, block_table, ctx.positions, ctx.tok_slot)
+    n = down.shape[0]
+    _need(down.dim() == 2 and n == ctx.n_tokens, f"{what}: rows {tuple(down.shape)} for {ctx.n_tokens} tokens")
+    _need(q_norm_w.shape == (q_rank,) and q_norm_w.dtype == F32 and kv_norm_w.shape == (kv_rank,) and kv_norm_w.dtype == F32,
+          f"{what}: the norms' weights are float32 [{q_rank}] and [{kv_rank}]")
+    _need(rows_cache.dim() == 3 and rows_cache.shape[1:] == (PAGE_TOKENS, kv_rank + rot_dim) and rows_cache.dtype == down.dtype,
+          f"{what}: the cache {tuple(rows_cache.shape)} {rows_cache.dtype} is not {down.dtype} [pages, {PAGE_TOKENS}, {kv_rank + rot_dim}]")
+    if rot_dim:
+        for tab in (cos, sin):
+            _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot_dim // 2), f"{what}: rotation rows are float32 [{n}, {rot_dim // 2}]")
+    _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
+    cq = torch.empty((n, q_rank), dtype=down.dtype, device=down.device)
+    library.call(mixers(), "palm_latent_prep", _stream(), _p(down), _code(down, what), down.shape[1], q_rank, kv_off, kv_rank, rot_dim,
+                 _p(q_norm_w), _p(kv_norm_w), float(eps), _p(cos), _p(sin), _p(ctx.positions), _p(ctx.tok_slot), _p(block_table),
+                 block_table.shape[1], _p(rows_cache), int(write_cache), _p(cq), n)
+    return cq
+
+
+def latent_query(q: torch.Tensor, uk: torch.Tensor, cos, sin, heads: int, dim: int, rot_dim: int, kv_rank: int) -> torch.Tensor:
+    """q [n, heads * (dim + rot_dim)], uk [heads * dim, kv_rank] -> float32 [n, heads, kv_rank + rot_dim]: each head's plain
+    part taken through its key matrix, its rotated part behind it."""
+    what = "latent_query"
+    _dev(what, q, uk, cos, sin)
+    n = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == heads * (dim + rot_dim) and uk.shape == (heads * dim, kv_rank),
+          f"{what}: q {tuple(q.shape)}, key matrix {tuple(uk.shape)} for {heads} heads of {dim} + {rot_dim} and a latent of {kv_rank}")
+    if rot_dim:
+        for tab in (cos, sin):
+            _need(tab is not None and tab.dtype == F32 and tab.shape == (n, rot_dim // 2), f"{what}: rotation rows are float32 [{n}, {rot_dim // 2}]")
+    qa = torch.empty((n, heads, kv_rank + rot_dim), dtype=F32, device=q.device)
+    library.call(mixers(), "palm_latent_query", _stream(), _p(q), _code(q, what), _p(uk), _code(uk, what + " key matrix"), _p(cos), _p(sin),
+                 n, heads, dim, rot_dim, kv_rank, _p(qa))
+    return qa
+
+
+def latent_attention(qa: torch.Tensor, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, heads: int, kv_rank: int,
+                     rot_dim: int, scale: float, window: int | None) -> torch.Tensor:
+    """Softmax attention of the step's queries (float32 [n, heads, kv_rank + rot_dim]) over the cached rows of their own
+    sequences up to their own positions (the last ``window`` of them if set): float32 [n, heads, kv_rank], the weighted sums
+    of the rows' latents."""
+    what = "latent_attention"
+    _dev(what, qa, rows_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    n = qa.shape[0]
+    _need(qa.shape == (n, heads, kv_rank + rot_dim) and qa.dtype == F32 and n == ctx.n_tokens, f"{what}: queries {tuple(qa.shape)} {qa.dtype}")
+    _need(rows_cache.dim() == 3 and rows_cache.shape[1:] == (PAGE_TOKENS, kv_rank + rot_dim),
+          f"{what}: the cache {tuple(rows_cache.shape)} is not [pages, {PAGE_TOKENS}, {kv_rank + rot_dim}]")
+    _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
+    out = torch.empty((n, heads, kv_rank), dtype=F32, device=qa.device)
+    library.call(mixers(), "palm_latent_attention", _stream(), _p(qa), _p(rows_cache), _code(rows_cache, what), _p(block_table),
+                 block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
+                 heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out))
+    return out
+
+
+def latent_output(o_lat: torch.Tensor, uv: torch.Tensor, gate: torch.Tensor | None, heads: int, kv_rank: int, vdim: int,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """o_lat float32 [n, heads, kv_rank], uv [heads * vdim, kv_rank], gate [n, heads] (a view of rows is fine) or None ->
+    [n, heads * vdim]: head h's latent sum through its value matrix, times sigmoid(gate[:, h])."""
+    what = "latent_output"
+    _dev(what, o_lat, uv)
+    n = o_lat.shape[0]
+    _need(o_lat.shape == (n, heads, kv_rank) and o_lat.dtype == F32 and uv.shape == (heads * vdim, kv_rank),
+          f"{what}: sums {tuple(o_lat.shape)} {o_lat.dtype}, value matrix {tuple(uv.shape)}")
+    _need(gate is None or (gate.is_cuda and gate.shape == (n, heads) and gate.dtype == out_dtype and (n == 0 or gate.stride(1) == 1)),
+          f"{what}: the gate is {out_dtype} [{n}, {heads}] with contiguous rows")
+    out = torch.empty((n, heads * vdim), dtype=out_dtype, device=o_lat.device)
+    library.call(mixers(), "palm_latent_output", _stream(), _p(o_lat), _p(uv), _code(uv, what + " value matrix"), _p(gate),
+                 gate.stride(0) if gate is not None else 0, _code(out, what), n, heads, kv_rank, vdim, _p(out))
+    return out
+
+
+# ---- routed experts ----------------------------------------------------------------------------------------------------
+
+def moe_route(logits: torch.Tensor, top: int):
+    """logits float32 [n, experts] -> (chosen int32 [n, top], weight float32 [n, top]): the ``top`` largest logits of each
+    row, largest first (the lower index wins a tie), and the softmax over them alone."""
+    _dev("moe_route", logits)
+    _need(logits.dim() == 2 and logits.dtype == F32, f"moe_route: router logits are float32 [n, experts], not {logits.dtype} {tuple(logits.shape)}")
+    n, experts = logits.shape
+    chosen = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((n, top), dtype=F32, device=logits.device)
+    library.call(mixers(), "palm_moe_route", _stream(), _p(logits), n, experts, int(top), _p(chosen), _p(weight))
+    return chosen, weight
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int) -> torch.Tensor:
+    """Every row through its chosen experts, nothing planned on the host: h [n, width]; gate_up [experts * 2 ff, width] (an
+    expert's gate rows, then its up rows); down [experts * width, ff].  Returns float32 [n, width], the weighted sum."""
+    what = "moe_experts"
+    _dev(what, h, gate_up, down, chosen, weight)
+    _i32(what, chosen)
+    n, width = h.shape
+    top = chosen.shape[1]
+    _need(gate_up.dim() == 2 and gate_up.shape[1] == width and gate_up.shape[0] % (2 * ff) == 0 and down.shape == (gate_up.shape[0] // (2 * ff) * width, ff)
+          and gate_up.dtype == down.dtype, f"{what}: gate/up {tuple(gate_up.shape)}, down {tuple(down.shape)} for width {width}, inner size {ff}")
+    _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == F32, f"{what}: choices {tuple(chosen.shape)}, weights {tuple(weight.shape)}")
+    mid = torch.empty((n, top, ff), dtype=F32, device=h.device)
+    out = torch.empty((n, width), dtype=F32, device=h.device)
+    library.call(mixers(), "palm_moe_experts", _stream(), _p(h), _code(h, what), _p(gate_up), _p(down), _code(gate_up, what + " weights"),
+                 _p(chosen), _p(weight), n, top, width, ff, _p(mid), _p(out))
+    return out
+
+
+def gather_rows(h: torch.Tensor, src: torch.Tensor) -> torch.Tensor:
+    """xs[p] = h[src[p]] (src int32)."""
+    _dev("gather_rows", h, src)
+    _i32("gather_rows", src)
+    _need(h.dim() == 2 and src.dim() == 1, f"gather_rows: rows {tuple(h.shape)}, indices {tuple(src.shape)}")
+    xs = torch.empty((src.shape[0], h.shape[1]), dtype=h.dtype, device=h.device)
+    library.call(mixers(), "palm_gather_rows", _stream(), _p(h), _code(h, "gather_rows"), _p(src), src.shape[0], h.shape[1], _p(xs))
+    return xs
+
+
+def scatter_add(out: torch.Tensor, y: torch.Tensor, rows: torch.Tensor, weight: torch.Tensor) -> None:
+    """out[rows[i]] += weight[i] * y[i]; out float32; the rows must be distinct."""
+    _dev("scatter_add", out, y, rows, weight)
+    _i32("scatter_add", rows)
+    _need(out.dtype == F32 and out.dim() == 2 and y.dim() == 2 and y.shape[1] == out.shape[1] and rows.shape == (y.shape[0],)
+          and weight.shape == (y.shape[0],) and weight.dtype == F32, f"scatter_add: out {tuple(out.shape)} {out.dtype}, y {tuple(y.shape)}, "
+          f"rows {tuple(rows.shape)}, weights {tuple(weight.shape)} {weight.dtype}")
+    library.call(mixers(), "palm_scatter_add", _stream(), _p(y), _code(y, "scatter_add"), _p(rows), _p(weight), y.shape[0], out.shape[1], _p(out))

@@ -2,7 +2,7 @@
 blocks, and the embedding and head at the two ends."""
 from .base import (CATEGORIES, Builder, StepContext, cache_needs, context_ints, make_context, part_class, register_part)
 from . import (norm, position, attention, feedforward, block, embedding, retention, selective_scan,  # noqa: F401  (registers the kinds)
-               differential_attention)
+               differential_attention, delta_rule, latent_attention)
 from .linear import Linear
 from .residual import Prenormed, ResidualSink, as_tensor, run_branch
 

@@ -12,6 +12,10 @@ branches read the stream itself (in the activation type).  A layer may have no f
 ``depth_weights`` c (float32 [J + 1]) the layer's result R_J = x is kept beside the earlier ones (R_0: the embedding
 rows) and what goes on is sum_j c[j] R_j: the model must say ``keeps_results``.  The norm, the add, the average and
 the rounded copy for the next reader are one kernel.
+
+``sandwich``: x += gain * norm_b(mixer(norm_a(x))); x += gain * norm_d(feed_forward(norm_c(x))): a norm on each side of
+every branch and one multiplier on what is added.  A layer may have no feed-forward.  The norm of a branch's output, the
+scaled add and the norm that reads the stream next are one kernel.
 """
 from __future__ import annotations
 
@@ -90,3 +94,49 @@ class PostNormBlock:
         if sink.rows is None and getattr(sink.norm, "passes_through", False):
             return h                                        # the next block reads the stream as it is
         return sink.norm(sink.x, rows=sink.rows)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock:
+    def __init__(self, spec, builder):
+        self.gain = float(spec.params.get("residual_gain", 1.0))
+        self.mixer_norm = builder.build(spec.parts["mixer_norm"])
+        self.mixer = builder.build(spec.parts["mixer"])
+        self.mixer_out_norm = builder.build(spec.parts["mixer_out_norm"])
+        self.feed_forward = builder.build(spec.parts["feed_forward"]) if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"]) if self.feed_forward is not None else None
+        self.feed_forward_out_norm = builder.build(spec.parts["feed_forward_out_norm"]) if self.feed_forward is not None else None
+        self.dtype = builder.dtype
+        for norm in (self.mixer_out_norm, self.feed_forward_out_norm):
+            if norm is not None and not getattr(norm, "folds_into_products", False):
+                raise ValueError("a sandwich block norms its branches' outputs with RMS norms")
+
+    @property
+    def capturable(self) -> bool:
+        parts = [self.mixer_norm, self.mixer, self.mixer_out_norm]
+        if self.feed_forward is not None:
+            parts += [self.feed_forward_norm, self.feed_forward, self.feed_forward_out_norm]
+        return all(getattr(p, "capturable", False) for p in parts)
+
+    @staticmethod
+    def cache_needs(spec):
+        return cache_needs(spec.parts["mixer"])
+
+    @property
+    def entry_norm(self):
+        return self.mixer_norm
+
+    def _add(self, x, y, out_norm, reader, rows):
+        """x += gain * out_norm(y); returns what ``reader`` (the norm that reads x next) makes of x, over ``rows``."""
+        if rows is None and getattr(reader, "folds_into_products", False):
+            return ops.add_normed_scaled(x, y, out_norm.weight, out_norm.eps, self.gain, reader.weight, reader.eps, self.dtype)
+        ops.add_normed_scaled(x, y, out_norm.weight, out_norm.eps, self.gain)
+        return reader(x, rows=rows)
+
+    def forward(self, x, h, ctx, sink):
+        y = self.mixer.forward(as_tensor(h), ctx)
+        if self.feed_forward is None:
+            return self._add(x, y, self.mixer_out_norm, sink.norm, sink.rows)
+        h = self._add(x, y, self.mixer_out_norm, self.feed_forward_norm, None)
+        y = self.feed_forward.forward(h, ctx)
+        return self._add(x, y, self.feed_forward_out_norm, sink.norm, sink.rows)

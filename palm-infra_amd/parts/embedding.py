@@ -12,17 +12,18 @@ from .linear import Linear
 class TokenEmbedding:
     capturable = True
 
-    """x[t, :] = E[id_t, :] widened to float32 (engine/engine.cpp:332-357).  Unlike the reference, an id
-    outside the table is not mapped to row 0: the step refuses it before anything runs."""
+    """x[t, :] = E[id_t, :] widened to float32 (engine/engine.cpp:332-357), times ``scale`` if the description gives
+    one.  Unlike the reference, an id outside the table is not mapped to row 0: the step refuses it before anything runs."""
 
     def __init__(self, spec, builder):
         self.table = builder.tensor(spec, "table")
         self.vocab, self.hidden = int(spec.params["vocab_size"]), int(spec.params["hidden_size"])
+        self.scale = float(spec.params.get("scale", 1.0))
         if self.table.shape != (self.vocab, self.hidden):
             raise ValueError(f"embedding table {tuple(self.table.shape)} is not [{self.vocab}, {self.hidden}]")
 
     def forward(self, token_ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-        return ops.embed(self.table, token_ids, out)
+        return ops.embed(self.table, token_ids, out, scale=self.scale)
 
 
 @register_part("head", "linear")
@@ -30,13 +31,15 @@ class LinearHead:
     capturable = True
 
     """logits = h W^T in float32; W is lm_head.weight, or the embedding table when the head is tied
-    (models/qwen3.py:89-95, 162-165; engine/engine.cpp:403-485)."""
+    (models/qwen3.py:89-95, 162-165; engine/engine.cpp:403-485).  With ``softcap`` c the logits are c * tanh(logits / c)."""
 
     def __init__(self, spec, builder):
         self.linear = Linear(builder.tensor(spec, "weight"))
         self.vocab = int(spec.params["vocab_size"])
+        self.softcap = float(spec.params["softcap"]) if spec.params.get("softcap") else None
         if self.linear.weight.shape != (self.vocab, int(spec.params["hidden_size"])):
             raise ValueError(f"head weight {tuple(self.linear.weight.shape)} does not fit")
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.linear(h, out_dtype=torch.float32)
+        logits = self.linear(h, out_dtype=torch.float32)
+        return ops.softcap(logits, self.softcap) if self.softcap else logits
