@@ -325,7 +325,8 @@ def other_sizes(name: str, args, sampler) -> dict:
 
 # ---- another design beside its closest relative -------------------------------------------------------------------
 # ``--design sebesun``: prompts and decode steps of the Sebesun presets (random weights) and of a Qwen3 model of the
-# same width, depth, head count and feed-forward width, with the time of every kernel entry point of one prompt step
+# same width, depth, head count and feed-forward width (``--design pazilorn``: the Pazilorn presets and the Sebesun presets
+# of the same width and depth), with the time of every kernel entry point of one prompt step
 # and one decode step (launched one by one under the kernel recorder), and for the mixers' kernels the fraction of the
 # peak that binds them.
 
@@ -350,6 +351,18 @@ def _mixer_rooflines(raw: dict, tokens: int, batch: int, context: int) -> dict:
                 kv = 2.0 * batch * context * m["kv_heads"] * (2 * m["dim"] + m["vdim"])
                 out["palm_attention_diff_mfma"] = (flops, mfma, None, None)
                 out["palm_attention_diff"] = (None, None, kv, hbm)
+            elif layer["type"] == "channel_delta" and "palm_delta_rule" not in out:
+                per = m["heads"] * m["dim"] * m["vdim"]                 # four multiply-adds for every element of S and token
+                out["palm_delta_rule"] = (8.0 * tokens * per, vec, 2.0 * 4 * batch * per, hbm)
+            elif layer["type"] == "latent_attention" and "palm_latent_attention" not in out:
+                w = m["mask"]["size"] if m.get("mask") else tokens
+                seen = sum(min(p + 1, w) for p in range(tokens))
+                row = m["kv_rank"] + m["rot_dim"]
+                out["palm_latent_attention"] = (2.0 * m["heads"] * (row + m["kv_rank"]) * seen, mfma,
+                                                2.0 * batch * min(context, w) * row, hbm)
+            if layer.get("mlp") and layer["mlp"].get("kind") == "moe" and "palm_moe_experts" not in out:
+                f = layer["mlp"]
+                out["palm_moe_experts"] = (None, None, 2.0 * batch * f["router"]["top"] * 3 * f["expert"]["ff"] * raw["width"], hbm)
     else:
         nh, nkv, hd = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
         out["palm_attention_prefill"] = (4.0 * nh * hd * pairs, mfma, None, None)
@@ -402,13 +415,7 @@ def design_points(raw: dict, args, tokens: int, batch: int, context: int) -> dic
             "kernels": table}
 
 
-def design_bench(args) -> int:
-    if args.design != "sebesun":
-        print(f"bench.py: --design {args.design}: only 'sebesun' is measured beside the default workload")
-        return 2
-    record = {"metric": "Sebesun presets beside Qwen3 models of equal width and depth: prompt and decode tok/s (bf16, random weights)",
-              "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
-              "data": "synthetic: random weights, uniform random token ids, no stop token", "sizes": {}}
+def _sebesun_bench(args, record) -> dict:
     for name in ("sebesun-2048", "sebesun-4096"):
         raw = preset_dict(name)
         att = next(layer["mixer"] for layer in raw["layers"] if layer["type"] == "attention")
@@ -420,7 +427,32 @@ def design_bench(args) -> int:
         record["sizes"][name] = {"sebesun": design_points(raw, args, PREFILL_TOKENS, BATCH, CONTEXT),
                                  "qwen3_twin": design_points(twin, args, PREFILL_TOKENS, BATCH, CONTEXT),
                                  "twin_config": sizes_text(twin)}
-    first = record["sizes"]["sebesun-2048"]["sebesun"]
+    return record["sizes"]["sebesun-2048"]["sebesun"]
+
+
+def _pazilorn_bench(args, record) -> dict:
+    """The Pazilorn presets beside the Sebesun presets of the same width and depth (the closest design here: a recurrence
+    with a state per head, attention with a value size of its own, layers with and without a feed-forward)."""
+    for width in ("2048", "4096"):
+        record["sizes"][f"pazilorn-{width}"] = {
+            "pazilorn": design_points(preset_dict(f"pazilorn-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT),
+            "sebesun": design_points(preset_dict(f"sebesun-{width}"), args, PREFILL_TOKENS, BATCH, CONTEXT)}
+    return record["sizes"]["pazilorn-2048"]["pazilorn"]
+
+
+DESIGNS = {"sebesun": ("Sebesun presets beside Qwen3 models of equal width and depth", _sebesun_bench),
+           "pazilorn": ("Pazilorn presets beside Sebesun presets of equal width and depth", _pazilorn_bench)}
+
+
+def design_bench(args) -> int:
+    if args.design not in DESIGNS:
+        print(f"bench.py: --design {args.design}: measured beside the default workload are {', '.join(sorted(DESIGNS))}")
+        return 2
+    title, run = DESIGNS[args.design]
+    record = {"metric": f"{title}: prompt and decode tok/s (bf16, random weights)",
+              "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
+              "data": "synthetic: random weights, uniform random token ids, no stop token", "sizes": {}}
+    first = run(args, record)
     record["value"], record["ms_per_step"] = first["decode_tps"], first["decode_ms"]
     print(json.dumps(record), flush=True)
     return 0
@@ -443,8 +475,8 @@ def main(argv=None) -> int:
     ap.add_argument("--only", default="8b,14b,32b", help="which sizes' points to measure (8b is always measured)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="tokens of the timed prompt (2,048 is the workload's; others serve profiles of longer prompts)")
-    ap.add_argument("--design", help="instead of the default workload: another design's presets beside a Qwen3 model of "
-                    "equal width and depth ('sebesun')")
+    ap.add_argument("--design", help="instead of the default workload: another design's presets beside its closest relative "
+                    "of equal width and depth ('sebesun' beside Qwen3, 'pazilorn' beside Sebesun)")
     args = ap.parse_args(argv)
     if args.design:
         if args.gpus != 1:

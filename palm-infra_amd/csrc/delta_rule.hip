@@ -106,23 +106,25 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ 
             float vn, bn, qn[QREGS], kn[QREGS], gn[QREGS];
             read_token(min(t0 + ti + 1, n_new - 1), vn, bn, qn, kn, gn);
             if (!mine) vv = 0.f;
-            float pred = 0.f;
+            // four partial sums each: the multiply-adds of a sum over d then wait for every fourth one before them only
+            float pr[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int d = 0; d < DMAX; ++d) {
                 const float gd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gv[d / WAVE]), d % WAVE));
                 const float kd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kv[d / WAVE]), d % WAVE));
                 S[d] *= gd;
-                pred = fmaf(S[d], kd, pred);
+                pr[d % 4] = fmaf(S[d], kd, pr[d % 4]);
             }
-            const float uu = bt * (vv - pred);
-            float acc = 0.f;
+            const float uu = bt * (vv - ((pr[0] + pr[1]) + (pr[2] + pr[3])));
+            float ac[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int d = 0; d < DMAX; ++d) {
                 const float qd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, qv[d / WAVE]), d % WAVE));
                 const float kd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kv[d / WAVE]), d % WAVE));
                 S[d] = fmaf(kd, uu, S[d]);
-                acc = fmaf(S[d], qd, acc);
+                ac[d % 4] = fmaf(S[d], qd, ac[d % 4]);
             }
+            const float acc = (ac[0] + ac[1]) + (ac[2] + ac[3]);
             o_s[ti][v] = acc;
             const float ss = wave_sum(acc * acc);
             if (lane == 0) red[ti][wave] = ss;

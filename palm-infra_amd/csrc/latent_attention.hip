@@ -19,6 +19,19 @@ constexpr int LAT_THREADS = 256;
 
 __device__ inline float lat_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// Eight neighbouring values of a row as floats: one 16-byte read of bfloat16, two of float32.
+__device__ inline void lat_load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 t = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
+    v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xffff0000u);
+}
+__device__ inline void lat_load8(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 // One block per token.  down: [n, stride] holding the query latent at 0 (q_rank), the key/value latent at kv_off
 // (kv_rank) and the key part to rotate behind it (rot_dim).  rows_cache: [pages, PAGE_TOKENS, kv_rank + rot_dim].
 template <typename T>
@@ -117,7 +130,7 @@ __global__ __launch_bounds__(LA_WAVES * WAVE) void latent_attention_kernel(
     const float* __restrict__ qa, const T* __restrict__ rows_cache, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_new,
     const int* __restrict__ cu_new, int heads, int kv_rank, int rot_dim, float scale, int window, float* __restrict__ out) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dk = kv_rank + rot_dim;
     float* q_s = lds;                                  // [HG][dk]
     float* acc_s = lds + HG * dk;                      // [HG][kv_rank]
@@ -155,10 +168,26 @@ __global__ __launch_bounds__(LA_WAVES * WAVE) void latent_attention_kernel(
         float s[HG];
 #pragma unroll
         for (int g = 0; g < HG; ++g) s[g] = 0.f;
-        for (int d = 0; d < dk; ++d) {
-            const float kd = to_float(kr[d]);
+        if (dk % 8 == 0) {                          // rows start on 16 bytes: eight values a read, the queries four a read
+            for (int d = 0; d < dk; d += 8) {
+                float kd[8];
+                lat_load8(kr + d, kd);
 #pragma unroll
-            for (int g = 0; g < HG; ++g) s[g] = fmaf(q_s[g * dk + d], kd, s[g]);
+                for (int g = 0; g < HG; ++g) {
+                    const float4 qa0 = *reinterpret_cast<const float4*>(q_s + g * dk + d);
+                    const float4 qa1 = *reinterpret_cast<const float4*>(q_s + g * dk + d + 4);
+                    s[g] = fmaf(qa0.x, kd[0], s[g]); s[g] = fmaf(qa0.y, kd[1], s[g]);
+                    s[g] = fmaf(qa0.z, kd[2], s[g]); s[g] = fmaf(qa0.w, kd[3], s[g]);
+                    s[g] = fmaf(qa1.x, kd[4], s[g]); s[g] = fmaf(qa1.y, kd[5], s[g]);
+                    s[g] = fmaf(qa1.z, kd[6], s[g]); s[g] = fmaf(qa1.w, kd[7], s[g]);
+                }
+            }
+        } else {
+            for (int d = 0; d < dk; ++d) {
+                const float kd = to_float(kr[d]);
+#pragma unroll
+                for (int g = 0; g < HG; ++g) s[g] = fmaf(q_s[g * dk + d], kd, s[g]);
+            }
         }
         float p[HG];
 #pragma unroll
@@ -223,15 +252,17 @@ __global__ __launch_bounds__(LA_WAVES * WAVE) void latent_attention_kernel(
     }
 }
 
-// One block per (tile of LO_TILE tokens, head): out[t, h, j] = sigmoid(gate[t, h]) * sum_r uv[h * vdim + j, r] * o_lat[t, h, r].
+// One block per (tile of LO_TILE tokens, head, group of LO_ROWS output rows):
+// out[t, h, j] = sigmoid(gate[t, h]) * sum_r uv[h * vdim + j, r] * o_lat[t, h, r].  A wave takes a row j at a time.
 constexpr int LO_TILE = 8;
+constexpr int LO_ROWS = 16;
 
 template <typename T, typename TW>
 __global__ __launch_bounds__(LAT_THREADS) void latent_output_kernel(
     const float* __restrict__ o_lat, const TW* __restrict__ uv, const T* __restrict__ gate, int gate_stride, int n_tokens,
     int heads, int kv_rank, int vdim, T* __restrict__ out) {
     extern __shared__ float lds[];                    // [LO_TILE][kv_rank]
-    const int t0 = blockIdx.x * LO_TILE, h = blockIdx.y;
+    const int t0 = blockIdx.x * LO_TILE, h = blockIdx.y, j0 = blockIdx.z * LO_ROWS;
     const int tt = min(LO_TILE, n_tokens - t0);
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = LAT_THREADS / WAVE;
     for (int idx = threadIdx.x; idx < LO_TILE * kv_rank; idx += LAT_THREADS) {
@@ -239,15 +270,26 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_output_kernel(
         lds[idx] = ti < tt ? o_lat[((size_t)(t0 + ti) * heads + h) * kv_rank + r] : 0.f;
     }
     __syncthreads();
-    for (int j = wave; j < vdim; j += n_waves) {
+    for (int j = j0 + wave; j < min(vdim, j0 + LO_ROWS); j += n_waves) {
         const TW* wr = uv + ((size_t)h * vdim + j) * kv_rank;
         float acc[LO_TILE];
 #pragma unroll
         for (int ti = 0; ti < LO_TILE; ++ti) acc[ti] = 0.f;
-        for (int r = lane; r < kv_rank; r += WAVE) {
-            const float wv = to_float(wr[r]);
+        if (kv_rank % 8 == 0) {
+            for (int r = lane * 8; r < kv_rank; r += WAVE * 8) {
+                float wv[8];
+                lat_load8(wr + r, wv);
 #pragma unroll
-            for (int ti = 0; ti < LO_TILE; ++ti) acc[ti] = fmaf(lds[ti * kv_rank + r], wv, acc[ti]);
+                for (int ti = 0; ti < LO_TILE; ++ti)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[ti] = fmaf(lds[ti * kv_rank + r + i], wv[i], acc[ti]);
+            }
+        } else {
+            for (int r = lane; r < kv_rank; r += WAVE) {
+                const float wv = to_float(wr[r]);
+#pragma unroll
+                for (int ti = 0; ti < LO_TILE; ++ti) acc[ti] = fmaf(lds[ti * kv_rank + r], wv, acc[ti]);
+            }
         }
 #pragma unroll
         for (int ti = 0; ti < LO_TILE; ++ti) {
@@ -333,9 +375,9 @@ PALM_API int palm_latent_output(hipStream_t stream, const float* o_lat, const vo
     PALM_CHECK(n_tokens >= 0 && heads > 0 && kv_rank > 0 && vdim > 0, "latent_output: n=%d heads=%d kv_rank=%d vdim=%d", n_tokens, heads,
                kv_rank, vdim);
     PALM_CHECK(kv_rank <= 1536, "latent_output: a latent of %d exceeds 1536", kv_rank);
-    PALM_CHECK(heads <= 65535, "latent_output: %d heads are more than one launch takes", heads);
+    PALM_CHECK(heads <= 65535 && vdim <= 65535 * LO_ROWS, "latent_output: %d heads of %d are more than one launch takes", heads, vdim);
     if (n_tokens == 0) return 0;
-    dim3 grid((n_tokens + LO_TILE - 1) / LO_TILE, heads);
+    dim3 grid((n_tokens + LO_TILE - 1) / LO_TILE, heads, (vdim + LO_ROWS - 1) / LO_ROWS);
     const size_t lds = (size_t)LO_TILE * kv_rank * sizeof(float);
     PALM_DTYPE_SWITCH(dtype, T, {
         PALM_DTYPE_SWITCH(w_dtype, TW, {

@@ -13,6 +13,19 @@
 
 constexpr int ROUTE_MAX_PER_LANE = 8;            // up to 512 experts
 
+// Eight neighbouring values of a row as floats: one 16-byte read of bfloat16, two of float32.
+__device__ inline void load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 t = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
+    v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xffff0000u);
+}
+__device__ inline void load8(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 // One wave per token.
 __global__ __launch_bounds__(WAVE) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
                                                          int* __restrict__ chosen, float* __restrict__ weight) {
@@ -70,10 +83,24 @@ __global__ __launch_bounds__(MOE_THREADS) void expert_gate_up_kernel(const T* __
         const TW* gr = w + (size_t)f * width;
         const TW* ur = w + (size_t)(ff + f) * width;
         float g = 0.f, u = 0.f;
-        for (int d = lane; d < width; d += WAVE) {
-            const float hv = h_s[d];
-            g = fmaf(to_float(gr[d]), hv, g);
-            u = fmaf(to_float(ur[d]), hv, u);
+        if (width % 8 == 0) {                       // rows start on 16 bytes: eight values a lane and read
+            for (int d = lane * 8; d < width; d += WAVE * 8) {
+                float gv[8], uv[8];
+                load8(gr + d, gv);
+                load8(ur + d, uv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float hv = h_s[d + i];
+                    g = fmaf(gv[i], hv, g);
+                    u = fmaf(uv[i], hv, u);
+                }
+            }
+        } else {
+            for (int d = lane; d < width; d += WAVE) {
+                const float hv = h_s[d];
+                g = fmaf(to_float(gr[d]), hv, g);
+                u = fmaf(to_float(ur[d]), hv, u);
+            }
         }
         g = wave_sum(g);
         u = wave_sum(u);
@@ -98,7 +125,16 @@ __global__ __launch_bounds__(MOE_THREADS) void expert_down_kernel(const float* _
         for (int c = 0; c < top; ++c) {
             const TW* wr = down + ((size_t)chosen[(size_t)t * top + c] * width + r) * ff;
             float acc = 0.f;
-            for (int f = lane; f < ff; f += WAVE) acc = fmaf(to_float(wr[f]), m_s[c * ff + f], acc);
+            if (ff % 8 == 0) {
+                for (int f = lane * 8; f < ff; f += WAVE * 8) {
+                    float wv[8];
+                    load8(wr + f, wv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc = fmaf(wv[i], m_s[c * ff + f + i], acc);
+                }
+            } else {
+                for (int f = lane; f < ff; f += WAVE) acc = fmaf(to_float(wr[f]), m_s[c * ff + f], acc);
+            }
             total = fmaf(weight[(size_t)t * top + c], wave_sum(acc), total);
         }
         if (lane == 0) out[(size_t)t * width + r] = total;

@@ -237,3 +237,11 @@ def forward(cfg: dict, t: dict, tokens, layers_out: list | None = None) -> torch
     logits = rms_norm(x, t["final.norm"], eps) @ t["embed"].T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+def greedy(cfg: dict, t: dict, prompt, n_new: int) -> list:
+    """The first maximum of the last position's logits, n_new times."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(torch.argmax(forward(cfg, t, ids)[-1])))
+    return ids[len(prompt):]
