@@ -18,6 +18,15 @@
 // A token's q, k and g are the same for every thread of the block: each wave reads the rows once, one value a lane,
 // and hands value d to all its lanes as a scalar operand.  A prompt and a single token run the same code, so a
 // prompt leaves the state that its tokens one by one leave.
+//
+// A long run of new tokens would keep only (heads x sequences) blocks busy, one token after the other.  A token's step is
+// linear in S: S_t = A_t S_(t-1) + beta_t k_t v_t^T with A_t = (I - beta_t k_t k_t^T) diag(g_t), so such a run is cut into
+// chunks of `chunk` tokens and done in three launches:
+//   1. every chunk alone: from a zero state with its values (its own sum L_c, [dim, vdim]), and from the identity with
+//      values of zero (the product P_c of its A_t, [dim, dim]: the same walk over dim more columns)       (all chunks at once)
+//   2. the chunks' starting states, one after the other: S_(c+1) = P_c S_c + L_c, S_0 the kept state      (small products)
+//   3. every chunk from its starting state, now with outputs                                             (all chunks at once)
+// The arithmetic of a token is the same in all three; only the order of the 32-bit sums over the past differs.
 #include "common.h"
 
 constexpr int DELTA_TILE = 8;
@@ -56,8 +65,15 @@ __global__ __launch_bounds__(WAVE) void delta_prep_kernel(const T* __restrict__ 
     if (lane == 0) beta[row * heads + h] = delta_sigmoid(to_float(b[row * b_stride + h]));
 }
 
+enum DeltaMode : int { DELTA_WHOLE = 0, DELTA_LOCAL = 1, DELTA_FROM_STARTS = 2 };
+
+// ext: [sequence x chunk][head][dim][vdim + dim]: a chunk's own sum beside the product of its steps (mode LOCAL writes
+// it: blockIdx.z = 0 the value columns, 1 the dim columns that start as the identity).  starts: [sequence x chunk][head]
+// [dim][vdim]: the states the chunks start from (mode FROM_STARTS reads them).
 template <typename T, int DMAX, int MAXT>
-__global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ u, int u_stride, int v_off,
+__global__ __launch_bounds__(MAXT) void delta_rule_kernel(int mode, int chunk, int max_chunks, float* __restrict__ ext,
+                                                          const float* __restrict__ starts,
+                                                          const T* __restrict__ u, int u_stride, int v_off,
                                                           const float* __restrict__ prep, const float* __restrict__ beta,
                                                           const float* __restrict__ gate, int gate_stride,
                                                           const float* __restrict__ norm_w, float eps,
@@ -67,22 +83,31 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ 
     __shared__ float red[DELTA_TILE][16];
     __shared__ float o_s[DELTA_TILE][MAXT];
     constexpr int QREGS = (DMAX + WAVE - 1) / WAVE;
-    const int h = blockIdx.x, b = blockIdx.y;
+    const int h = blockIdx.x, b = blockIdx.y / max_chunks, c = blockIdx.y % max_chunks;
+    const bool steps_part = blockIdx.z == 1;                     // the columns that become the product of the chunk's steps
     const int v = threadIdx.x;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
-    const int n_new = seq_new[b];
-    if (n_new <= 0) return;
-    const int row0 = cu_new[b];
-    const bool mine = v < vdim;
+    const int seq_tokens = seq_new[b];
+    if (seq_tokens <= 0 || (mode != DELTA_WHOLE && c * chunk >= seq_tokens)) return;
+    const int n_new = mode == DELTA_WHOLE ? seq_tokens : min(chunk, seq_tokens - c * chunk);
+    const int row0 = cu_new[b] + (mode == DELTA_WHOLE ? 0 : c * chunk);
+    const int cols = steps_part ? dim : vdim;
+    const bool mine = v < cols;
     const int vc = min(v, vdim - 1);
-    float* sp = state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + vc;
 
     // unconditional reads of rows and a column that exist; what does not belong is set to zero after
     float S[DMAX];
+    if (mode == DELTA_LOCAL) {
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-        const float s0 = sp[(size_t)min(d, dim - 1) * vdim];
-        S[d] = (!mine || d >= dim) ? 0.f : s0;
+        for (int d = 0; d < DMAX; ++d) S[d] = (steps_part && mine && d == v) ? 1.f : 0.f;
+    } else {
+        const float* sp = mode == DELTA_WHOLE ? state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + vc
+                                              : starts + ((((size_t)b * max_chunks + c) * heads + h) * dim) * vdim + vc;
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d) {
+            const float s0 = sp[(size_t)min(d, dim - 1) * vdim];
+            S[d] = (!mine || d >= dim) ? 0.f : s0;
+        }
     }
 
     auto read_token = [&](int t, float& vv, float& bt, float (&qv)[QREGS], float (&kv)[QREGS], float (&gv)[QREGS]) {
@@ -105,7 +130,7 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ 
         for (int ti = 0; ti < tt; ++ti) {                        // not unrolled: the body is 2 DMAX steps long already
             float vn, bn, qn[QREGS], kn[QREGS], gn[QREGS];
             read_token(min(t0 + ti + 1, n_new - 1), vn, bn, qn, kn, gn);
-            if (!mine) vv = 0.f;
+            if (!mine || steps_part) vv = 0.f;
             // four partial sums each: the multiply-adds of a sum over d then wait for every fourth one before them only
             float pr[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -125,14 +150,17 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ 
                 ac[d % 4] = fmaf(S[d], qd, ac[d % 4]);
             }
             const float acc = (ac[0] + ac[1]) + (ac[2] + ac[3]);
-            o_s[ti][v] = acc;
-            const float ss = wave_sum(acc * acc);
-            if (lane == 0) red[ti][wave] = ss;
+            if (mode != DELTA_LOCAL) {
+                o_s[ti][v] = acc;
+                const float ss = wave_sum(acc * acc);
+                if (lane == 0) red[ti][wave] = ss;
+            }
             vv = vn;
             bt = bn;
 #pragma unroll
             for (int c = 0; c < QREGS; ++c) { qv[c] = qn[c]; kv[c] = kn[c]; gv[c] = gn[c]; }
         }
+        if (mode == DELTA_LOCAL) continue;
         __syncthreads();
         for (int ti = 0; ti < tt; ++ti) {
             float total = 0.f;
@@ -144,11 +172,82 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(const T* __restrict__ 
         }
         __syncthreads();
     }
-    if (mine) {
+    if (mine && mode == DELTA_WHOLE) {
+        float* sp = state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim + v;
 #pragma unroll
         for (int d = 0; d < DMAX; ++d)
             if (d < dim) sp[(size_t)d * vdim] = S[d];
     }
+    if (mine && mode == DELTA_LOCAL) {
+        const int ev = vdim + dim;
+        float* ep = ext + ((((size_t)b * max_chunks + c) * heads + h) * dim) * ev + (steps_part ? vdim : 0) + v;
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d)
+            if (d < dim) ep[(size_t)d * ev] = S[d];
+    }
+}
+
+// Step 2 above.  One block per (head, sequence, tile of 64 value columns): the tile of S lies in LDS; for every chunk the
+// block first hands the chunk its starting state, then makes S <- P_c S + L_c: a wave takes rows of the result, four at a
+// time (a read of S from LDS serves four multiply-adds), a lane a column; the row of P_c is the same for all lanes.
+constexpr int DS_WAVES = 8;
+
+__global__ __launch_bounds__(DS_WAVES * WAVE) void delta_starts_kernel(const float* __restrict__ ext, float* __restrict__ starts,
+                                                                       float* __restrict__ state, const int* __restrict__ seq_slot,
+                                                                       const int* __restrict__ seq_new, int chunk, int max_chunks,
+                                                                       int heads, int dim, int vdim) {
+    extern __shared__ float s_s[];                      // [dim][WAVE]
+    const int h = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * WAVE;
+    const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int n_new = seq_new[b];
+    if (n_new <= 0) return;
+    const int v = v0 + lane;
+    const bool mine = v < vdim;
+    const int vc = min(v, vdim - 1), ev = vdim + dim;
+    float* st = state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim;
+    for (int d = wave; d < dim; d += DS_WAVES) s_s[d * WAVE + lane] = mine ? st[(size_t)d * vdim + vc] : 0.f;
+    __syncthreads();
+    for (int c = 0; c * chunk < n_new; ++c) {
+        const size_t at = (((size_t)b * max_chunks + c) * heads + h) * dim;
+        const float* ep = ext + at * ev;
+        float* sc = starts + at * vdim;
+        float fresh[8][4];                              // this wave's rows of the new state: up to 32 rows (dim up to 256)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            const int d0 = (n * DS_WAVES + wave) * 4;
+            if (d0 >= dim) continue;                    // (the same for the whole wave)
+            float acc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = ep[(size_t)min(d0 + i, dim - 1) * ev + vc];           // L_c
+            const float* p0 = ep + (size_t)min(d0, dim - 1) * ev + vdim;
+            const float* p1 = ep + (size_t)min(d0 + 1, dim - 1) * ev + vdim;
+            const float* p2 = ep + (size_t)min(d0 + 2, dim - 1) * ev + vdim;
+            const float* p3 = ep + (size_t)min(d0 + 3, dim - 1) * ev + vdim;
+            for (int e = 0; e < dim; ++e) {
+                const float se = s_s[e * WAVE + lane];
+                acc[0] = fmaf(p0[e], se, acc[0]);
+                acc[1] = fmaf(p1[e], se, acc[1]);
+                acc[2] = fmaf(p2[e], se, acc[2]);
+                acc[3] = fmaf(p3[e], se, acc[3]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fresh[n][i] = acc[i];
+        }
+        // the chunk starts from the state as it was
+        for (int d = wave; d < dim; d += DS_WAVES)
+            if (mine) sc[(size_t)d * vdim + v] = s_s[d * WAVE + lane];
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            const int d0 = (n * DS_WAVES + wave) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (d0 + i < dim) s_s[(d0 + i) * WAVE + lane] = fresh[n][i];
+        }
+        __syncthreads();
+    }
+    for (int d = wave; d < dim; d += DS_WAVES)
+        if (mine) st[(size_t)d * vdim + v] = s_s[d * WAVE + lane];
 }
 
 PALM_API int palm_delta_pad(int dim) { return dim <= 32 ? 32 : dim <= 64 ? 64 : dim <= 128 ? 128 : 256; }
@@ -157,36 +256,51 @@ PALM_API int palm_delta_pad(int dim) { return dim <= 32 ? 32 : dim <= 64 ? 64 : 
 // b: the write strengths before the sigmoid, [n, b_stride] of the same type, one a head; a: float32 [n, a_stride], the
 // decays' rows before bias and softplus (heads * dim); gate: float32 [n, gate_stride], the output gate before the
 // sigmoid (heads * vdim).  prep: room for n * heads * 3 * palm_delta_pad(dim) floats, beta_buf: n * heads floats.
+// chunk == 0: every sequence's run in one block per head.  Else, with max_chunks = ceil(max_new / chunk): ext holds
+// n_seqs * max_chunks * heads * dim * (vdim + dim) floats and starts n_seqs * max_chunks * heads * dim * vdim.
 PALM_API int palm_delta_rule(hipStream_t stream, const void* u, int dtype, int u_stride, int q_off, int k_off, int v_off,
                              const void* b, int b_stride, const float* a, int a_stride, const float* gate, int gate_stride,
                              const float* a_log, const float* dt_bias, const float* norm_w, float q_scale, float unit_eps,
                              float eps, float* state, const int* seq_slot, const int* seq_new, const int* cu_new, int n_seqs,
-                             int heads, int kv_heads, int dim, int vdim, void* out, int n_tokens, float* prep, float* beta_buf) {
+                             int heads, int kv_heads, int dim, int vdim, void* out, int n_tokens, float* prep, float* beta_buf,
+                             int max_new, int chunk, float* ext, float* starts) {
     PALM_CHECK(n_seqs >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "delta_rule: seqs=%d heads=%d kv=%d dim=%d vdim=%d",
                n_seqs, heads, kv_heads, dim, vdim);
     PALM_CHECK(heads % kv_heads == 0, "delta_rule: %d heads are not a multiple of %d q/k heads", heads, kv_heads);
     PALM_CHECK(dim <= 256, "delta_rule: a key size of %d exceeds 256", dim);
     PALM_CHECK(vdim <= 1024, "delta_rule: a value size of %d exceeds 1024", vdim);
     PALM_CHECK(n_tokens >= 0 && (n_tokens == 0 || (prep && beta_buf)), "delta_rule: the prepared rows need their room");
+    PALM_CHECK(chunk >= 0 && (chunk == 0 || (ext && starts && max_new > 0)), "delta_rule: chunks of %d tokens need room for their sums, "
+               "products and starting states", chunk);
     if (n_seqs == 0 || n_tokens == 0) return 0;
-    PALM_CHECK(heads <= 65535 && n_seqs <= 65535, "delta_rule: %d heads / %d sequences are more than one launch takes", heads, n_seqs);
-    const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
+    const int max_chunks = chunk > 0 ? (max_new + chunk - 1) / chunk : 1;
+    PALM_CHECK(heads <= 65535 && (long long)n_seqs * max_chunks <= 65535, "delta_rule: %d heads / %d sequences x %d chunks are more than one "
+               "launch takes", heads, n_seqs, max_chunks);
     const int pad = palm_delta_pad(dim);
-    dim3 grid(heads, n_seqs);
-#define DELTA_CASE(D) { if (threads <= 256) delta_rule_kernel<T, D, 256><<<grid, threads, 0, stream>>>((const T*)u, u_stride, v_off, prep, \
-            beta_buf, gate, gate_stride, norm_w, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out); \
-        else delta_rule_kernel<T, D, 1024><<<grid, threads, 0, stream>>>((const T*)u, u_stride, v_off, prep, \
-            beta_buf, gate, gate_stride, norm_w, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out); }
+    const int threads = (vdim + WAVE - 1) / WAVE * WAVE;
+    const int local_threads = (max(vdim, dim) + WAVE - 1) / WAVE * WAVE;
+    dim3 grid(heads, n_seqs * max_chunks);
+#define DELTA_LAUNCH(D, GRID, THREADS, MODE) { if ((THREADS) <= 256) delta_rule_kernel<T, D, 256><<<GRID, THREADS, 0, stream>>>(MODE, chunk, max_chunks, \
+            ext, starts, (const T*)u, u_stride, v_off, prep, beta_buf, gate, gate_stride, norm_w, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out); \
+        else delta_rule_kernel<T, D, 1024><<<GRID, THREADS, 0, stream>>>(MODE, chunk, max_chunks, \
+            ext, starts, (const T*)u, u_stride, v_off, prep, beta_buf, gate, gate_stride, norm_w, eps, state, seq_slot, seq_new, cu_new, heads, dim, vdim, (T*)out); }
+#define DELTA_CASE(GRID, THREADS, MODE) { if (dim <= 32) DELTA_LAUNCH(32, GRID, THREADS, MODE) else if (dim <= 64) DELTA_LAUNCH(64, GRID, THREADS, MODE) \
+        else if (dim <= 128) DELTA_LAUNCH(128, GRID, THREADS, MODE) else DELTA_LAUNCH(256, GRID, THREADS, MODE) }
     PALM_DTYPE_SWITCH(dtype, T, {
         delta_prep_kernel<T><<<dim3(n_tokens, heads), WAVE, 0, stream>>>((const T*)u, u_stride, q_off, k_off, (const T*)b, b_stride, a,
                                                                         a_stride, a_log, dt_bias, q_scale, unit_eps, heads, kv_heads,
                                                                         dim, pad, prep, beta_buf);
-        if (dim <= 32) DELTA_CASE(32)
-        else if (dim <= 64) DELTA_CASE(64)
-        else if (dim <= 128) DELTA_CASE(128)
-        else DELTA_CASE(256)
+        if (chunk == 0) {
+            DELTA_CASE(grid, threads, DELTA_WHOLE)
+        } else {
+            DELTA_CASE(dim3(heads, n_seqs * max_chunks, 2), local_threads, DELTA_LOCAL)
+            delta_starts_kernel<<<dim3(heads, n_seqs, (vdim + WAVE - 1) / WAVE), DS_WAVES * WAVE, (size_t)dim * WAVE * sizeof(float), stream>>>(
+                ext, starts, state, seq_slot, seq_new, chunk, max_chunks, heads, dim, vdim);
+            DELTA_CASE(grid, threads, DELTA_FROM_STARTS)
+        }
     });
 #undef DELTA_CASE
+#undef DELTA_LAUNCH
     PALM_LAUNCHED();
     return 0;
 }

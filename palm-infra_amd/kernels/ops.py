@@ -781,7 +781,7 @@ _MIXER_SIGNATURES = {
     "palm_delta_pad": [c_int],
     "palm_delta_rule": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                         c_void_p, c_void_p, c_void_p, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                        c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p],
+                        c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "palm_latent_prep": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p,
                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int],
     "palm_latent_query": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -1088,16 +1088,33 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 # ---- the delta rule ------------------------------------------------------------------------------------------------
 
+DELTA_BLOCKS_WANTED = 512          # a long run of new tokens is cut into chunks until about this many blocks run
+DELTA_MIN_CHUNK = 64
+
+
+def delta_chunk(n_seqs: int, heads: int, max_new: int) -> int:
+    """Into chunks of how many tokens the delta rule's kernel cuts the step's runs of new tokens (0: not at all).  One block
+    per (head, sequence) walks over its tokens one after the other; where that leaves most of the chip idle and the runs
+    are long, chunks run side by side at the price of walking over every token twice, over the key size more columns the
+    first time, and of a small product for every chunk between the two walks."""
+    per_seq = DELTA_BLOCKS_WANTED // max(1, heads * n_seqs)
+    if max_new <= 2 * DELTA_MIN_CHUNK or per_seq <= 1:
+        return 0
+    chunk = max(DELTA_MIN_CHUNK, -(-max_new // per_seq))
+    chunk = (chunk + 7) // 8 * 8
+    return chunk if chunk < max_new else 0
+
+
 def delta_rule(u: torch.Tensor, offsets: tuple, b: torch.Tensor, a: torch.Tensor, gate: torch.Tensor, a_log: torch.Tensor,
                dt_bias: torch.Tensor, norm_w: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, q_scale: float,
-               unit_eps: float, eps: float, state: torch.Tensor, ctx) -> torch.Tensor:
+               unit_eps: float, eps: float, state: torch.Tensor, ctx, chunk: int | None = None) -> torch.Tensor:
     """The step's tokens through the recurrence of a gated delta rule with one decay per key channel.
 
     u [n, >= 2 kv_heads dim + heads vdim]: the convolution's output with q, k, v at the columns ``offsets``; b [n, heads]
     (a view of rows is fine: its row stride is passed on): the write strengths before the sigmoid; a float32 [n, heads * dim]
     and gate float32 [n, heads * vdim] (views likewise): the decays' rows before bias and softplus, the output gate before
     its sigmoid; state float32 [slots, heads, dim, vdim], read and left updated.  Returns [n, heads * vdim]: the heads'
-    outputs, each normed over vdim with ``norm_w`` and gated."""
+    outputs, each normed over vdim with ``norm_w`` and gated.  ``chunk``: see ``delta_chunk`` (None: chosen here)."""
     what = "delta_rule"
     _dev(what, u, a_log, dt_bias, norm_w, state, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
     _i32(what, ctx.seq_slot, ctx.seq_new, ctx.cu_new)
@@ -1115,10 +1132,16 @@ def delta_rule(u: torch.Tensor, offsets: tuple, b: torch.Tensor, a: torch.Tensor
     out = torch.empty((n, heads * vdim), dtype=u.dtype, device=u.device)
     prep = torch.empty((n, heads, 3, mixers().palm_delta_pad(dim)), dtype=F32, device=u.device)
     beta = torch.empty((n, heads), dtype=F32, device=u.device)
+    chunk = delta_chunk(ctx.n_seqs, heads, ctx.max_new) if chunk is None else int(chunk)
+    ext = starts = None
+    if chunk:
+        chunks = ctx.n_seqs * (-(-ctx.max_new // chunk))
+        ext = torch.empty((chunks, heads, dim, vdim + dim), dtype=F32, device=u.device)
+        starts = torch.empty((chunks, heads, dim, vdim), dtype=F32, device=u.device)
     library.call(mixers(), "palm_delta_rule", _stream(), _p(u), _code(u, what), u.stride(0), q_off, k_off, v_off, _p(b), b.stride(0),
                  _p(a), a.stride(0), _p(gate), gate.stride(0), _p(a_log), _p(dt_bias), _p(norm_w), float(q_scale), float(unit_eps),
                  float(eps), _p(state), _p(ctx.seq_slot), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, heads, kv_heads, dim, vdim,
-                 _p(out), n, _p(prep), _p(beta))
+                 _p(out), n, _p(prep), _p(beta), int(ctx.max_new), chunk, _p(ext), _p(starts))
     return out
 
 

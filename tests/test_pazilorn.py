@@ -346,6 +346,8 @@ def _delta_plain(c, heads, kv, dim, vdim, eps, drop_first=False):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv,dim,vdim", [(2, 1, 12, 20), (3, 3, 40, 72), (1, 1, 96, 130), (2, 2, 130, 64)])
 def test_delta_rule_kernel_keeps_a_far_write_whole_and_in_portions(dtype, heads, kv, dim, vdim):
+    """Whole, in portions down to two tokens and single tokens, and cut by the kernel into chunks that run side by side (of
+    a size given here, 0 for none, or of its own choice): the outputs and the state left behind."""
     from palm_infra_amd.kernels import ops
     T, eps = 300, 1e-5
     c = _delta_case(T, heads, kv, dim, vdim, dtype, seed=dim + vdim)
@@ -354,7 +356,8 @@ def test_delta_rule_kernel_keeps_a_far_write_whole_and_in_portions(dtype, heads,
     assert float((want[-1] - without[-1]).abs().max()) > 0.3            # the far write decides the last output
     dev = {k: v.cuda() for k, v in c.items()}
     tol = dict(atol=2e-4, rtol=1e-4) if dtype == "float32" else dict(atol=0.03, rtol=0.03)
-    for portions in ([T], [150, 64, 5, 2, 79], [1] * 3 + [T - 3]):
+    for portions, chunk in (([T], 0), ([150, 64, 5, 2, 79], 0), ([1] * 3 + [T - 3], 0), ([T], 32), ([T], 64), ([T], 104), ([130, 170], 48),
+                            ([T], None)):
         state = torch.full((3, heads, dim, vdim), float("nan"), device="cuda")
         state[1] = 0.0                                                   # slot 1 is the sequence's; its neighbours hold rubbish
         got, lo = [], 0
@@ -363,10 +366,10 @@ def test_delta_rule_kernel_keeps_a_far_write_whole_and_in_portions(dtype, heads,
             sl = slice(lo, lo + n)
             got.append(ops.delta_rule(dev["u"][sl].contiguous(), (0, kv * dim, 2 * kv * dim), dev["b"][sl].contiguous(), dev["a"][sl].contiguous(),
                                       dev["gate"][sl].contiguous(), dev["a_log"], dev["dt_bias"], dev["norm_w"], heads, kv, dim, vdim,
-                                      dim ** -0.5, 1e-6, eps, state, ctx))
+                                      dim ** -0.5, 1e-6, eps, state, ctx, chunk=chunk))
             lo += n
         got = torch.cat(got).double().cpu()
-        assert torch.allclose(got, want, **tol), f"portions {portions}: {float((got - want).abs().max())}"
+        assert torch.allclose(got, want, **tol), f"portions {portions}, chunks of {chunk}: {float((got - want).abs().max())}"
         assert torch.allclose(state[1].double().cpu(), want_state, atol=1e-4 if dtype == "float32" else 1e-3, rtol=1e-3)
         assert torch.isnan(state[0]).all() and torch.isnan(state[2]).all()
 
