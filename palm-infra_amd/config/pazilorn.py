@@ -123,6 +123,9 @@ class PazilornConfig:
         out["scale"] = _get(m, "scale", float, where)
         if out["rot_dim"] < 0 or out["rot_dim"] % 2:
             raise ConfigError(f"config.json: {where}.rot_dim = {out['rot_dim']} must be even and not negative")
+        if out["kv_rank"] > 1024 or out["kv_rank"] + out["rot_dim"] > 1280 or out["dim"] > 512:
+            raise ConfigError(f"config.json: {where}: the attention kernels take latents up to 1024 (with the rotated part 1280) and "
+                              "unrotated key sizes up to 512")
         mask = m.get("mask")
         out["mask"] = {"size": _positive(_get(mask, "size", int, where + ".mask"), where + ".mask.size")} if mask else None
         rot = m.get("rot")

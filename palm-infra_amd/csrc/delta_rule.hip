@@ -187,67 +187,69 @@ __global__ __launch_bounds__(MAXT) void delta_rule_kernel(int mode, int chunk, i
     }
 }
 
-// Step 2 above.  One block per (head, sequence, tile of 64 value columns): the tile of S lies in LDS; for every chunk the
-// block first hands the chunk its starting state, then makes S <- P_c S + L_c: a wave takes rows of the result, four at a
-// time (a read of S from LDS serves four multiply-adds), a lane a column; the row of P_c is the same for all lanes.
+// Step 2 above.  One block per (head, sequence, tile of DS_COLS value columns): the tile of S lies in LDS.  For every chunk
+// the block first hands the chunk its starting state, then makes S <- P_c S + L_c: a thread owns one column of the tile and
+// every 32nd row of the result (a quarter of a wave a column run, 8 waves x 4 quarters = 32 row groups), reads its rows of
+// P_c four values at a time and S from LDS.
 constexpr int DS_WAVES = 8;
+constexpr int DS_COLS = 16;
+constexpr int DS_GROUPS = DS_WAVES * (WAVE / DS_COLS);          // 32 row groups
+constexpr int DS_MAX_ROWS = 256 / DS_GROUPS;                    // rows a thread owns at most (dim up to 256)
 
 __global__ __launch_bounds__(DS_WAVES * WAVE) void delta_starts_kernel(const float* __restrict__ ext, float* __restrict__ starts,
                                                                        float* __restrict__ state, const int* __restrict__ seq_slot,
                                                                        const int* __restrict__ seq_new, int chunk, int max_chunks,
                                                                        int heads, int dim, int vdim) {
-    extern __shared__ float s_s[];                      // [dim][WAVE]
-    const int h = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * WAVE;
-    const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    extern __shared__ __attribute__((aligned(16))) float s_s[];         // [dim][DS_COLS]
+    const int h = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * DS_COLS;
+    const int col = threadIdx.x % DS_COLS, group = threadIdx.x / DS_COLS;
     const int n_new = seq_new[b];
     if (n_new <= 0) return;
-    const int v = v0 + lane;
+    const int v = v0 + col;
     const bool mine = v < vdim;
     const int vc = min(v, vdim - 1), ev = vdim + dim;
     float* st = state + (((size_t)seq_slot[b] * heads + h) * dim) * vdim;
-    for (int d = wave; d < dim; d += DS_WAVES) s_s[d * WAVE + lane] = mine ? st[(size_t)d * vdim + vc] : 0.f;
+    for (int d = group; d < dim; d += DS_GROUPS) s_s[d * DS_COLS + col] = mine ? st[(size_t)d * vdim + vc] : 0.f;
     __syncthreads();
     for (int c = 0; c * chunk < n_new; ++c) {
         const size_t at = (((size_t)b * max_chunks + c) * heads + h) * dim;
         const float* ep = ext + at * ev;
         float* sc = starts + at * vdim;
-        float fresh[8][4];                              // this wave's rows of the new state: up to 32 rows (dim up to 256)
+        float fresh[DS_MAX_ROWS];
 #pragma unroll
-        for (int n = 0; n < 8; ++n) {
-            const int d0 = (n * DS_WAVES + wave) * 4;
-            if (d0 >= dim) continue;                    // (the same for the whole wave)
-            float acc[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = ep[(size_t)min(d0 + i, dim - 1) * ev + vc];           // L_c
-            const float* p0 = ep + (size_t)min(d0, dim - 1) * ev + vdim;
-            const float* p1 = ep + (size_t)min(d0 + 1, dim - 1) * ev + vdim;
-            const float* p2 = ep + (size_t)min(d0 + 2, dim - 1) * ev + vdim;
-            const float* p3 = ep + (size_t)min(d0 + 3, dim - 1) * ev + vdim;
-            for (int e = 0; e < dim; ++e) {
-                const float se = s_s[e * WAVE + lane];
-                acc[0] = fmaf(p0[e], se, acc[0]);
-                acc[1] = fmaf(p1[e], se, acc[1]);
-                acc[2] = fmaf(p2[e], se, acc[2]);
-                acc[3] = fmaf(p3[e], se, acc[3]);
+        for (int i = 0; i < DS_MAX_ROWS; ++i) {
+            const int d = group + i * DS_GROUPS;
+            const int dc = min(d, dim - 1);
+            const float* pr = ep + (size_t)dc * ev + vdim;              // row d of P_c (16-byte reads where the rows allow them)
+            float acc = ep[(size_t)dc * ev + vc];                       // L_c
+            if (d < dim) {
+                if (ev % 4 == 0 && vdim % 4 == 0 && dim % 4 == 0) {
+                    for (int e = 0; e < dim; e += 4) {
+                        const float4 p = *reinterpret_cast<const float4*>(pr + e);
+                        acc = fmaf(p.x, s_s[e * DS_COLS + col], acc);
+                        acc = fmaf(p.y, s_s[(e + 1) * DS_COLS + col], acc);
+                        acc = fmaf(p.z, s_s[(e + 2) * DS_COLS + col], acc);
+                        acc = fmaf(p.w, s_s[(e + 3) * DS_COLS + col], acc);
+                    }
+                } else {
+                    for (int e = 0; e < dim; ++e) acc = fmaf(pr[e], s_s[e * DS_COLS + col], acc);
+                }
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fresh[n][i] = acc[i];
+            fresh[i] = acc;
         }
         // the chunk starts from the state as it was
-        for (int d = wave; d < dim; d += DS_WAVES)
-            if (mine) sc[(size_t)d * vdim + v] = s_s[d * WAVE + lane];
+        for (int d = group; d < dim; d += DS_GROUPS)
+            if (mine) sc[(size_t)d * vdim + v] = s_s[d * DS_COLS + col];
         __syncthreads();
 #pragma unroll
-        for (int n = 0; n < 8; ++n) {
-            const int d0 = (n * DS_WAVES + wave) * 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (d0 + i < dim) s_s[(d0 + i) * WAVE + lane] = fresh[n][i];
+        for (int i = 0; i < DS_MAX_ROWS; ++i) {
+            const int d = group + i * DS_GROUPS;
+            if (d < dim) s_s[d * DS_COLS + col] = fresh[i];
         }
         __syncthreads();
     }
-    for (int d = wave; d < dim; d += DS_WAVES)
-        if (mine) st[(size_t)d * vdim + v] = s_s[d * WAVE + lane];
+    for (int d = group; d < dim; d += DS_GROUPS)
+        if (mine) st[(size_t)d * vdim + v] = s_s[d * DS_COLS + col];
 }
 
 PALM_API int palm_delta_pad(int dim) { return dim <= 32 ? 32 : dim <= 64 ? 64 : dim <= 128 ? 128 : 256; }
@@ -294,7 +296,7 @@ PALM_API int palm_delta_rule(hipStream_t stream, const void* u, int dtype, int u
             DELTA_CASE(grid, threads, DELTA_WHOLE)
         } else {
             DELTA_CASE(dim3(heads, n_seqs * max_chunks, 2), local_threads, DELTA_LOCAL)
-            delta_starts_kernel<<<dim3(heads, n_seqs, (vdim + WAVE - 1) / WAVE), DS_WAVES * WAVE, (size_t)dim * WAVE * sizeof(float), stream>>>(
+            delta_starts_kernel<<<dim3(heads, n_seqs, (vdim + DS_COLS - 1) / DS_COLS), DS_WAVES * WAVE, (size_t)dim * DS_COLS * sizeof(float), stream>>>(
                 ext, starts, state, seq_slot, seq_new, chunk, max_chunks, heads, dim, vdim);
             DELTA_CASE(grid, threads, DELTA_FROM_STARTS)
         }

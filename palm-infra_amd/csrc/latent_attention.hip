@@ -72,48 +72,53 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_prep_kernel(
     }
 }
 
-// One block per (tile of LQ_TILE tokens, head).  q: [n, heads * (dim + rot_dim)], a head's plain part first.
-// uk: [heads * dim, kv_rank].  qa: float32 [n, heads, kv_rank + rot_dim].
+// One block per (tile of LQ_TILE tokens, head, run of LQ_COLS latent columns).  q: [n, heads * (dim + rot_dim)], a head's
+// plain part first.  uk: [heads * dim, kv_rank].  qa: float32 [n, heads, kv_rank + rot_dim].  A thread owns a column of
+// the key matrix and walks down it (neighbouring threads read neighbouring values); the first run's block also rotates.
 constexpr int LQ_TILE = 8;
+constexpr int LQ_COLS = 64;
 constexpr int LQ_MAX_DIM = 512;
 
 template <typename T, typename TW>
-__global__ __launch_bounds__(LAT_THREADS) void latent_query_kernel(
+__global__ __launch_bounds__(LQ_COLS) void latent_query_kernel(
     const T* __restrict__ q, const TW* __restrict__ uk, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     int n_tokens, int heads, int dim, int rot_dim, int kv_rank, float* __restrict__ qa) {
     __shared__ float q_s[LQ_TILE][LQ_MAX_DIM];
     const int t0 = blockIdx.x * LQ_TILE, h = blockIdx.y;
     const int tt = min(LQ_TILE, n_tokens - t0);
     const int hd = dim + rot_dim, dk = kv_rank + rot_dim, half = rot_dim / 2;
-    for (int idx = threadIdx.x; idx < LQ_TILE * dim; idx += LAT_THREADS) {
+    for (int idx = threadIdx.x; idx < LQ_TILE * dim; idx += LQ_COLS) {
         const int ti = idx / dim, d = idx % dim;
         q_s[ti][d] = ti < tt ? to_float(q[((size_t)(t0 + ti) * heads + h) * hd + d]) : 0.f;
     }
-    for (int idx = threadIdx.x; idx < tt * half; idx += LAT_THREADS) {
-        const int ti = idx / half, i = idx % half;
-        const size_t row = t0 + ti;
-        const T* qr = q + (row * heads + h) * hd + dim;
-        const float c = cos_t[row * half + i], s = sin_t[row * half + i];
-        const float a = to_float(qr[i]), b = to_float(qr[half + i]);
-        float* o = qa + (row * heads + h) * dk + kv_rank;
-        o[i] = a * c - b * s;
-        o[half + i] = b * c + a * s;
+    if (blockIdx.z == 0) {
+        for (int idx = threadIdx.x; idx < tt * half; idx += LQ_COLS) {
+            const int ti = idx / half, i = idx % half;
+            const size_t row = t0 + ti;
+            const T* qr = q + (row * heads + h) * hd + dim;
+            const float c = cos_t[row * half + i], s = sin_t[row * half + i];
+            const float a = to_float(qr[i]), b = to_float(qr[half + i]);
+            float* o = qa + (row * heads + h) * dk + kv_rank;
+            o[i] = a * c - b * s;
+            o[half + i] = b * c + a * s;
+        }
     }
     __syncthreads();
     const TW* w = uk + (size_t)h * dim * kv_rank;
-    for (int r = threadIdx.x; r < kv_rank; r += LAT_THREADS) {
-        float acc[LQ_TILE];
+    const int r = blockIdx.z * LQ_COLS + threadIdx.x;
+    if (r >= kv_rank) return;
+    float acc[LQ_TILE];
 #pragma unroll
-        for (int ti = 0; ti < LQ_TILE; ++ti) acc[ti] = 0.f;
-        for (int d = 0; d < dim; ++d) {
-            const float wv = to_float(w[(size_t)d * kv_rank + r]);
+    for (int ti = 0; ti < LQ_TILE; ++ti) acc[ti] = 0.f;
+#pragma unroll 4
+    for (int d = 0; d < dim; ++d) {
+        const float wv = to_float(w[(size_t)d * kv_rank + r]);
 #pragma unroll
-            for (int ti = 0; ti < LQ_TILE; ++ti) acc[ti] = fmaf(q_s[ti][d], wv, acc[ti]);
-        }
-#pragma unroll
-        for (int ti = 0; ti < LQ_TILE; ++ti)
-            if (ti < tt) qa[((size_t)(t0 + ti) * heads + h) * dk + r] = acc[ti];
+        for (int ti = 0; ti < LQ_TILE; ++ti) acc[ti] = fmaf(q_s[ti][d], wv, acc[ti]);
     }
+#pragma unroll
+    for (int ti = 0; ti < LQ_TILE; ++ti)
+        if (ti < tt) qa[((size_t)(t0 + ti) * heads + h) * dk + r] = acc[ti];
 }
 
 // One block of LA_WAVES waves per (query, group of HG heads).  A wave takes every LA_WAVES-th page of the key range;
@@ -252,17 +257,19 @@ __global__ __launch_bounds__(LA_WAVES * WAVE) void latent_attention_kernel(
     }
 }
 
-// One block per (tile of LO_TILE tokens, head, group of LO_ROWS output rows):
-// out[t, h, j] = sigmoid(gate[t, h]) * sum_r uv[h * vdim + j, r] * o_lat[t, h, r].  A wave takes a row j at a time.
+// One block per (tile of LO_TILE tokens, head, group of `rows` output rows):
+// out[t, h, j] = sigmoid(gate[t, h]) * sum_r uv[h * vdim + j, r] * o_lat[t, h, r].  A wave takes a row j at a time.  A
+// step of few tokens cuts a head's rows into groups of 16 so that blocks enough run; a prompt's blocks take all rows of a
+// head (the tile's sums are brought into LDS once).
 constexpr int LO_TILE = 8;
-constexpr int LO_ROWS = 16;
+constexpr int LO_FEW_ROWS = 16;
 
 template <typename T, typename TW>
 __global__ __launch_bounds__(LAT_THREADS) void latent_output_kernel(
     const float* __restrict__ o_lat, const TW* __restrict__ uv, const T* __restrict__ gate, int gate_stride, int n_tokens,
-    int heads, int kv_rank, int vdim, T* __restrict__ out) {
+    int heads, int kv_rank, int vdim, int rows, T* __restrict__ out) {
     extern __shared__ float lds[];                    // [LO_TILE][kv_rank]
-    const int t0 = blockIdx.x * LO_TILE, h = blockIdx.y, j0 = blockIdx.z * LO_ROWS;
+    const int t0 = blockIdx.x * LO_TILE, h = blockIdx.y, j0 = blockIdx.z * rows;
     const int tt = min(LO_TILE, n_tokens - t0);
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = LAT_THREADS / WAVE;
     for (int idx = threadIdx.x; idx < LO_TILE * kv_rank; idx += LAT_THREADS) {
@@ -270,12 +277,12 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_output_kernel(
         lds[idx] = ti < tt ? o_lat[((size_t)(t0 + ti) * heads + h) * kv_rank + r] : 0.f;
     }
     __syncthreads();
-    for (int j = j0 + wave; j < min(vdim, j0 + LO_ROWS); j += n_waves) {
+    for (int j = j0 + wave; j < min(vdim, j0 + rows); j += n_waves) {
         const TW* wr = uv + ((size_t)h * vdim + j) * kv_rank;
         float acc[LO_TILE];
 #pragma unroll
         for (int ti = 0; ti < LO_TILE; ++ti) acc[ti] = 0.f;
-        if (kv_rank % 8 == 0) {
+        if (kv_rank % 8 == 0 && kv_rank >= WAVE * 8) {            // (a shorter row: a value a lane keeps all lanes busy)
             for (int r = lane * 8; r < kv_rank; r += WAVE * 8) {
                 float wv[8];
                 lat_load8(wr + r, wv);
@@ -330,10 +337,10 @@ PALM_API int palm_latent_query(hipStream_t stream, const void* q, int dtype, con
     PALM_CHECK(rot_dim == 0 || (cos_t && sin_t), "latent_query: a rotation needs its cos and sin rows");
     PALM_CHECK(heads <= 65535, "latent_query: %d heads are more than one launch takes", heads);
     if (n_tokens == 0) return 0;
-    dim3 grid((n_tokens + LQ_TILE - 1) / LQ_TILE, heads);
+    dim3 grid((n_tokens + LQ_TILE - 1) / LQ_TILE, heads, (kv_rank + LQ_COLS - 1) / LQ_COLS);
     PALM_DTYPE_SWITCH(dtype, T, {
         PALM_DTYPE_SWITCH(w_dtype, TW, {
-            latent_query_kernel<T, TW><<<grid, LAT_THREADS, 0, stream>>>((const T*)q, (const TW*)uk, cos_t, sin_t, n_tokens, heads, dim,
+            latent_query_kernel<T, TW><<<grid, LQ_COLS, 0, stream>>>((const T*)q, (const TW*)uk, cos_t, sin_t, n_tokens, heads, dim,
                                                                         rot_dim, kv_rank, qa);
         });
     });
@@ -375,14 +382,15 @@ PALM_API int palm_latent_output(hipStream_t stream, const float* o_lat, const vo
     PALM_CHECK(n_tokens >= 0 && heads > 0 && kv_rank > 0 && vdim > 0, "latent_output: n=%d heads=%d kv_rank=%d vdim=%d", n_tokens, heads,
                kv_rank, vdim);
     PALM_CHECK(kv_rank <= 1536, "latent_output: a latent of %d exceeds 1536", kv_rank);
-    PALM_CHECK(heads <= 65535 && vdim <= 65535 * LO_ROWS, "latent_output: %d heads of %d are more than one launch takes", heads, vdim);
+    PALM_CHECK(heads <= 65535 && vdim <= 65535 * LO_FEW_ROWS, "latent_output: %d heads of %d are more than one launch takes", heads, vdim);
     if (n_tokens == 0) return 0;
-    dim3 grid((n_tokens + LO_TILE - 1) / LO_TILE, heads, (vdim + LO_ROWS - 1) / LO_ROWS);
+    const int rows = n_tokens <= 64 ? LO_FEW_ROWS : vdim;
+    dim3 grid((n_tokens + LO_TILE - 1) / LO_TILE, heads, (vdim + rows - 1) / rows);
     const size_t lds = (size_t)LO_TILE * kv_rank * sizeof(float);
     PALM_DTYPE_SWITCH(dtype, T, {
         PALM_DTYPE_SWITCH(w_dtype, TW, {
-            latent_output_kernel<T, TW><<<grid, LAT_THREADS, lds, stream>>>(o_lat, (const TW*)uv, (const T*)gate, gate_stride, n_tokens,
-                                                                           heads, kv_rank, vdim, (T*)out);
+            latent_output_kernel<T, TW><<<grid, LAT_THREADS, lds, stream>>>(o_lat, (const TW*)uv, (const T*)gate, gate_stride, n_tokens, heads,
+                                                                           kv_rank, vdim, rows, (T*)out);
         });
     });
     PALM_LAUNCHED();
