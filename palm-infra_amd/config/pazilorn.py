@@ -118,7 +118,9 @@ class PazilornConfig:
                 if m.get(k) is not None:
                     out[k] = _positive(int(m[k]), f"{where}.{k}")
             return out
-        out = {k: _positive(_get(m, k, int, where), f"{where}.{k}") for k in ("heads", "dim", "vdim", "kv_rank", "q_rank")}
+        out = {k: _positive(_get(m, k, int, where), f"{where}.{k}") for k in ("heads", "dim", "vdim", "kv_rank")}
+        if m.get("q_rank") is not None:              # else the rows of the query's down projection give it
+            out["q_rank"] = _positive(int(m["q_rank"]), f"{where}.q_rank")
         out["rot_dim"] = _get(m, "rot_dim", int, where)
         out["scale"] = _get(m, "scale", float, where)
         if out["rot_dim"] < 0 or out["rot_dim"] % 2:
@@ -157,17 +159,17 @@ class PazilornConfig:
         return {"kind": kind, "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
 
     def with_tensor_shapes(self, shapes: dict) -> "PazilornConfig":
-        """The configuration with the sizes that only a checkpoint's tensors give: the ranks of the delta rule's low-rank
-        pairs (rows of ``l<i>.mix.a1`` and ``l<i>.mix.g1``)."""
+        """The configuration with the sizes that a checkpoint's tensors give: the ranks of the delta rule's low-rank pairs
+        (rows of ``l<i>.mix.a1`` and ``l<i>.mix.g1``) and of the attention's query latent (rows of ``l<i>.mix.dq``)."""
         layers = []
         for i, layer in enumerate(self.layers):
-            if layer["type"] == "channel_delta":
-                j = self._source(self.layers, i)
-                m = dict(layer["mixer"])
-                for key, name in (("decay_rank", f"l{j}.mix.a1"), ("gate_rank", f"l{j}.mix.g1")):
-                    if name in shapes and len(shapes[name]) == 2:
-                        m[key] = int(shapes[name][0])
-                layer = dict(layer, mixer=m)
+            j = self._source(self.layers, i)
+            m = dict(layer["mixer"])
+            given = (("decay_rank", f"l{j}.mix.a1"), ("gate_rank", f"l{j}.mix.g1")) if layer["type"] == "channel_delta" else (("q_rank", f"l{j}.mix.dq"),)
+            for key, name in given:
+                if name in shapes and len(shapes[name]) == 2:
+                    m[key] = int(shapes[name][0])
+            layer = dict(layer, mixer=m)
             layers.append(layer)
         return replace(self, layers=tuple(layers))
 
@@ -202,6 +204,8 @@ class PazilornConfig:
                  "dt_bias": tensor(p + "dt_bias", (H * d,), "vector", ("normal", -1.0, 1.0)),
                  "norm": tensor(p + "norm", (dv,), "vector", _NORM_INIT),
                  "out": tensor(p + "o", (W, H * dv))})
+        if "q_rank" not in m:
+            raise ConfigError(f"layers[{i}].mixer: the rank of the query's latent is given by q_rank or by the shape of {p}dq")
         H, d, dr, dv, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
         parts = {}
         if m["rot"] is not None:

@@ -62,7 +62,6 @@ class LatentAttention:
         down = self.down(h)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
-        dr = self.dr if tables is not None else 0
         cq = ops.latent_prep(down, self.q_rank, self.q_rank, self.kv_rank, self.dr, self.q_norm_w, self.kv_norm_w, self.eps, cos, sin,
                              view.data, view.table_dev, ctx, write_cache=lc.writes)
         qa = ops.latent_query(self.uq(cq), self.uk, cos, sin, self.nh, self.dk, self.dr, self.kv_rank)

@@ -56,8 +56,17 @@ CONFIGS = {
           "embedding": {"scale": 12.0}, "logit_softcap": None, "layers": [
               _with(_latent(2, 8, 4, 12, 70, 16, 0.5, None, 250000.0, {"factor": 16.0, "original": 32, "fast": 4.0, "slow": 2.0}), 16, 9, 1),
           ]},
+    # larger sizes: a key size of two waves' worth of registers, more experts than a wave has lanes, a latent of several
+    # values a lane with one head a block, heads that fill no group, a window of several pages, borrowed weights named ahead
+    "D": {"architecture": "Pazilorn", "vocab": 150, "width": 96, "norm": {"eps": 1e-5}, "residual_mult": 0.3,
+          "embedding": {"scale": 10.0}, "logit_softcap": 12.0, "layers": [
+              _with(_latent(5, 32, 16, 48, 136, 72, 0.2, 130, 50000.0, {"factor": 8.0, "original": 128, "fast": 16.0, "slow": 1.0}), 24, 70, 5, weights_of=2),
+              _with(_delta(4, 1, 128, 64, 3, 8, 8), 48, 4, 2),
+              _with(_latent(5, 32, 16, 48, 136, 72, 0.2, 130, 50000.0, {"factor": 8.0, "original": 128, "fast": 16.0, "slow": 1.0}), 24, 70, 5),
+              _with(_latent(2, 16, 2, 8, 600, 40, 0.3, 9, 100.0), None),
+          ]},
 }
-SEEDS = {"A": 31, "B": 32, "C": 33}
+SEEDS = {"A": 31, "B": 32, "C": 33, "D": 34}
 # one layer of one kind, for the tests of a mechanism alone
 SINGLE = {
     "channel_delta": {"architecture": "Pazilorn", "vocab": 90, "width": 32, "norm": {"eps": 1e-6}, "residual_mult": 1.0,
@@ -85,16 +94,16 @@ def sharpened_tensors(raw: dict, seed: int, store: str) -> dict:
 
 
 def write_model(raw: dict, seed: int, path, store: str, drop_ranks: bool = True) -> Path:
-    """A model folder.  ``drop_ranks``: config.json does not give the low ranks, as a checkpoint's configuration does not:
-    the tensors' shapes do."""
+    """A model folder.  ``drop_ranks``: config.json does not give the delta rule's low ranks, as a checkpoint's configuration
+    does not (and for some of the configurations not the query latent's either): the tensors' shapes do."""
     path = Path(path)
     path.mkdir(parents=True, exist_ok=True)
     tensors = sharpened_tensors(raw, seed, store)
     if drop_ranks:
         raw = json.loads(json.dumps(raw))
         for layer in raw["layers"]:
-            layer["mixer"].pop("decay_rank", None)
-            layer["mixer"].pop("gate_rank", None)
+            for key in ("decay_rank", "gate_rank") + (("q_rank",) if raw["width"] % 32 == 0 else ()):      # (q_rank: in some of them)
+                layer["mixer"].pop(key, None)
     (path / "config.json").write_text(json.dumps(raw))
     write_safetensors(path / "model.safetensors", tensors)
     return path

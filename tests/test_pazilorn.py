@@ -21,7 +21,7 @@ from palm_infra_amd.config import ConfigError, config_from_dict
 
 gpu = pytest.mark.gpu
 DTYPES = ("float32", "bfloat16")
-LENGTHS = {"A": [1, 2, 63, 64, 65, 130, 200, 17], "B": [129, 3, 70, 71, 1, 191], "C": [5, 66, 128, 31]}
+LENGTHS = {"A": [1, 2, 63, 64, 65, 130, 200, 17], "B": [129, 3, 70, 71, 1, 191], "C": [5, 66, 128, 31], "D": [300, 9, 140]}
 
 
 # ---- without a GPU ---------------------------------------------------------------------------------------
@@ -236,7 +236,7 @@ class Pool:
         assert_close(torch.cat(self.got), torch.cat(self.ref), self.dtype, self.what + " (all rows together)")
 
 
-CASES = [(n, d) for n in ("A", "B", "C") for d in DTYPES]
+CASES = [(n, d) for n in ("A", "B", "C", "D") for d in DTYPES]
 
 
 def _step_context(lengths_before, new_counts, slots=None):
@@ -657,7 +657,7 @@ def test_recorded_and_launched_steps_agree(tmp_path_factory, name):
 
 
 @gpu
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_greedy_generation_through_generate(tmp_path_factory, name):
     from palm_infra_amd.sampling import GREEDY
     eng = engine_for(tmp_path_factory, name, "float32")
