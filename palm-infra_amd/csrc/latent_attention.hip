@@ -9,7 +9,8 @@
 // expanded, all heads read the same rows.  Scores, softmax and sums are 32-bit.
 //
 //   latent_prep        the joined down projection's rows -> the normed query latent; the normed latent and the
-//                      rotated key part into the position's cache row
+//                      rotated key part into the position's cache row (and, where the caller keeps one for the prompt
+//                      kernel of latent_attention_mfma.hip, the latent into a bfloat16 copy with the positions innermost)
 //   latent_query       q rows -> [a_h | rotated q_rot,h] per head, 32-bit
 //   latent_attention   softmax over the visible rows (causal, optional window), o_lat,h = sum_j p_j c_j, 32-bit
 //   latent_output      head h: sigmoid(gate_h) * U_v,h o_lat,h
@@ -39,7 +40,8 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_prep_kernel(
     const T* __restrict__ down, int stride, int q_rank, int kv_off, int kv_rank, int rot_dim, const float* __restrict__ q_norm_w,
     const float* __restrict__ kv_norm_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, const int* __restrict__ block_table, int max_pages,
-    T* __restrict__ rows_cache, int write_cache, T* __restrict__ cq) {
+    T* __restrict__ rows_cache, int write_cache, T* __restrict__ cq, bf16_t* __restrict__ rows_t,
+    const int* __restrict__ block_table_t) {
     __shared__ float scratch[16];
     const size_t row = blockIdx.x;
     const T* dr = down + row * stride;
@@ -63,6 +65,12 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_prep_kernel(
     const int page = block_table[(size_t)tok_slot[row] * max_pages + pos / PAGE_TOKENS];
     T* cr = rows_cache + ((size_t)page * PAGE_TOKENS + pos % PAGE_TOKENS) * (kv_rank + rot_dim);
     for (int d = threadIdx.x; d < kv_rank; d += LAT_THREADS) cr[d] = from_float<T>((to_float(dr[kv_off + d]) * ki) * kv_norm_w[d]);
+    if (rows_t) {                                   // the latent once more, positions innermost: [pages, kv_rank, PAGE_TOKENS]
+        const int page_t = block_table_t[(size_t)tok_slot[row] * max_pages + pos / PAGE_TOKENS];
+        bf16_t* ct = rows_t + (size_t)page_t * kv_rank * PAGE_TOKENS + pos % PAGE_TOKENS;
+        for (int d = threadIdx.x; d < kv_rank; d += LAT_THREADS)
+            ct[(size_t)d * PAGE_TOKENS] = f32_to_bf16((to_float(dr[kv_off + d]) * ki) * kv_norm_w[d]);
+    }
     const int half = rot_dim / 2;
     for (int i = threadIdx.x; i < half; i += LAT_THREADS) {
         const float c = cos_t[row * half + i], s = sin_t[row * half + i];
@@ -313,18 +321,20 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_output_kernel(
 PALM_API int palm_latent_prep(hipStream_t stream, const void* down, int dtype, int stride, int q_rank, int kv_off, int kv_rank,
                               int rot_dim, const float* q_norm_w, const float* kv_norm_w, float eps, const float* cos_t,
                               const float* sin_t, const int* positions, const int* tok_slot, const int* block_table, int max_pages,
-                              void* rows_cache, int write_cache, void* cq, int n_tokens) {
+                              void* rows_cache, int write_cache, void* cq, int n_tokens, void* rows_t, const int* block_table_t) {
     PALM_CHECK(n_tokens >= 0 && q_rank > 0 && kv_rank > 0 && rot_dim >= 0 && rot_dim % 2 == 0, "latent_prep: n=%d q_rank=%d kv_rank=%d rot_dim=%d",
                n_tokens, q_rank, kv_rank, rot_dim);
     PALM_CHECK(stride >= kv_off + kv_rank + rot_dim && kv_off >= q_rank, "latent_prep: rows of %d do not hold %d + %d + %d", stride, q_rank,
                kv_rank, rot_dim);
     PALM_CHECK(rot_dim == 0 || (cos_t && sin_t), "latent_prep: a rotation needs its cos and sin rows");
     PALM_CHECK(max_pages > 0, "latent_prep: max_pages %d", max_pages);
+    PALM_CHECK(!rows_t || block_table_t, "latent_prep: the transposed copy needs its page table");
     if (n_tokens == 0) return 0;
     PALM_DTYPE_SWITCH(dtype, T,
         latent_prep_kernel<T><<<n_tokens, LAT_THREADS, 0, stream>>>((const T*)down, stride, q_rank, kv_off, kv_rank, rot_dim, q_norm_w,
                                                                    kv_norm_w, eps, cos_t, sin_t, positions, tok_slot, block_table,
-                                                                   max_pages, (T*)rows_cache, write_cache, (T*)cq));
+                                                                   max_pages, (T*)rows_cache, write_cache, (T*)cq, (bf16_t*)rows_t,
+                                                                   block_table_t));
     PALM_LAUNCHED();
     return 0;
 }

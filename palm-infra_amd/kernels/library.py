@@ -13,6 +13,8 @@ Libraries:
                         scan and its convolution, differential attention, the delta rule, attention over compressed
                         rows), routed experts, and the stream of blocks that norm a branch's output; loaded when a
                         model has such a part
+  ``latent_attention_k<K>_v<V>``  attention over compressed rows for prompts on the matrix cores, compiled for rows up to
+                        32 K and latents up to 16 V
   ``attention_diff_k<K>_v<V>_q<Q>``  differential attention for prompts on the matrix cores, compiled for key sizes up to
                         32 K, value sizes up to 16 V and Q tiles of 16 queries a wave
 """
@@ -45,6 +47,7 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
 DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
+LATENT_ATTENTION_SOURCES = ["latent_attention_mfma.hip"]
 MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
                  "latent_attention.hip", "moe.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
@@ -178,6 +181,9 @@ def _spec(name: str):
         kk, rest = name[len("attention_diff_k"):].split("_v")
         vt, qt = rest.split("_q")
         return DIFF_ATTENTION_SOURCES, (f"PALM_DIFF_KK={int(kk)}", f"PALM_DIFF_VT={int(vt)}", f"PALM_DIFF_QT={int(qt)}")
+    if name.startswith("latent_attention_k"):
+        kk, vt = name[len("latent_attention_k"):].split("_v")
+        return LATENT_ATTENTION_SOURCES, (f"PALM_LAT_KK={int(kk)}", f"PALM_LAT_VT={int(vt)}")
     if name.startswith("attention_hd"):
         hd = int(name[len("attention_hd"):])
         return ATTENTION_SOURCES, (f"PALM_HEAD_DIM={hd}",)

@@ -783,7 +783,7 @@ _MIXER_SIGNATURES = {
                         c_void_p, c_void_p, c_void_p, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                         c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "palm_latent_prep": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p,
-                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int],
+                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p],
     "palm_latent_query": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "palm_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -1148,13 +1148,18 @@ def delta_rule(u: torch.Tensor, offsets: tuple, b: torch.Tensor, a: torch.Tensor
 # ---- attention over one compressed row per position -----------------------------------------------------------------
 
 def latent_prep(down: torch.Tensor, q_rank: int, kv_off: int, kv_rank: int, rot_dim: int, q_norm_w, kv_norm_w, eps: float,
-                cos, sin, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, write_cache: bool = True) -> torch.Tensor:
+                cos, sin, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, write_cache: bool = True,
+                rows_t: torch.Tensor | None = None, table_t: torch.Tensor | None = None) -> torch.Tensor:
     """down [n, >= kv_off + kv_rank + rot_dim]: the query latent at column 0, the key/value latent at ``kv_off`` and the key
     part to rotate behind it.  Returns the normed query latent [n, q_rank]; writes [normed latent | rotated key part] into
-    each token's row of ``rows_cache`` [pages, PAGE_TOKENS, kv_rank + rot_dim]."""
+    each token's row of ``rows_cache`` [pages, PAGE_TOKENS, kv_rank + rot_dim] and, if given, the normed latent into
+    ``rows_t`` (bfloat16 [pages, kv_rank, PAGE_TOKENS], with the page table ``table_t`` of its own)."""
     what = "latent_prep"
-    _dev(what, down, q_norm_w, kv_norm_w, cos, sin, rows_cache, block_table, ctx.positions, ctx.tok_slot)
-    _i32(what, block_table, ctx.positions, ctx.tok_slot)
+    _dev(what, down, q_norm_w, kv_norm_w, cos, sin, rows_cache, block_table, ctx.positions, ctx.tok_slot, rows_t, table_t)
+    _i32(what, block_table, ctx.positions, ctx.tok_slot, table_t)
+    _need(rows_t is None or (table_t is not None and rows_t.dtype == BF16 and rows_t.dim() == 3 and rows_t.shape[1:] == (kv_rank, PAGE_TOKENS)
+                             and table_t.shape == block_table.shape),
+          f"{what}: the transposed copy is bfloat16 [pages, {kv_rank}, {PAGE_TOKENS}] with a page table like the rows'")
     n = down.shape[0]
     _need(down.dim() == 2 and n == ctx.n_tokens, f"{what}: rows {tuple(down.shape)} for {ctx.n_tokens} tokens")
     _need(q_norm_w.shape == (q_rank,) and q_norm_w.dtype == F32 and kv_norm_w.shape == (kv_rank,) and kv_norm_w.dtype == F32,
@@ -1168,7 +1173,7 @@ def latent_prep(down: torch.Tensor, q_rank: int, kv_off: int, kv_rank: int, rot_
     cq = torch.empty((n, q_rank), dtype=down.dtype, device=down.device)
     library.call(mixers(), "palm_latent_prep", _stream(), _p(down), _code(down, what), down.shape[1], q_rank, kv_off, kv_rank, rot_dim,
                  _p(q_norm_w), _p(kv_norm_w), float(eps), _p(cos), _p(sin), _p(ctx.positions), _p(ctx.tok_slot), _p(block_table),
-                 block_table.shape[1], _p(rows_cache), int(write_cache), _p(cq), n)
+                 block_table.shape[1], _p(rows_cache), int(write_cache), _p(cq), n, _p(rows_t), _p(table_t))
     return cq
 
 
@@ -1189,20 +1194,55 @@ def latent_query(q: torch.Tensor, uk: torch.Tensor, cos, sin, heads: int, dim: i
     return qa
 
 
+_LATENT_MFMA_SIGNATURE = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]
+_latent_libs: dict = {}
+LATENT_MFMA_MAX_ROW, LATENT_MFMA_MAX_RANK = 640, 512
+
+
+def latent_mfma_serves(rows_cache: torch.Tensor, kv_rank: int, rot_dim: int) -> bool:
+    """The matrix-core kernel takes bfloat16 rows whose sizes are multiples of eight, up to 640 values a row and a latent of 512."""
+    return (rows_cache.dtype == BF16 and kv_rank % 8 == 0 and (kv_rank + rot_dim) % 8 == 0 and kv_rank + rot_dim <= LATENT_MFMA_MAX_ROW
+            and kv_rank <= LATENT_MFMA_MAX_RANK)
+
+
+def latent_attention_lib(kv_rank: int, rot_dim: int):
+    key = ((kv_rank + rot_dim + 31) // 32, (kv_rank + 15) // 16)
+    if key not in _latent_libs:
+        lib = library.load(f"latent_attention_k{key[0]}_v{key[1]}")
+        lib.palm_latent_attention_mfma.argtypes, lib.palm_latent_attention_mfma.restype = _LATENT_MFMA_SIGNATURE, c_int
+        lib.palm_latent_attention_mfma_sizes.argtypes, lib.palm_latent_attention_mfma_sizes.restype = [c_int], c_int
+        if tuple(lib.palm_latent_attention_mfma_sizes(i) for i in range(2)) != (key[0] * 32, key[1] * 16):
+            raise KernelError(f"library latent_attention_k{key[0]}_v{key[1]} was built for other sizes")
+        _latent_libs[key] = lib
+    return _latent_libs[key]
+
+
 def latent_attention(qa: torch.Tensor, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, heads: int, kv_rank: int,
-                     rot_dim: int, scale: float, window: int | None) -> torch.Tensor:
+                     rot_dim: int, scale: float, window: int | None, rows_t: torch.Tensor | None = None,
+                     table_t: torch.Tensor | None = None) -> torch.Tensor:
     """Softmax attention of the step's queries (float32 [n, heads, kv_rank + rot_dim]) over the cached rows of their own
     sequences up to their own positions (the last ``window`` of them if set): float32 [n, heads, kv_rank], the weighted sums
-    of the rows' latents."""
+    of the rows' latents.  Prompts (and portions of them) in bfloat16 go to the matrix cores if the caller keeps the
+    transposed copy of the latents (``rows_t`` [pages, kv_rank, PAGE_TOKENS] with its page table); single tokens, the
+    float32 mode and sizes that kernel does not take go to the exact kernel."""
     what = "latent_attention"
-    _dev(what, qa, rows_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
-    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new)
+    _dev(what, qa, rows_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new, rows_t, table_t)
+    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new, table_t)
     n = qa.shape[0]
     _need(qa.shape == (n, heads, kv_rank + rot_dim) and qa.dtype == F32 and n == ctx.n_tokens, f"{what}: queries {tuple(qa.shape)} {qa.dtype}")
     _need(rows_cache.dim() == 3 and rows_cache.shape[1:] == (PAGE_TOKENS, kv_rank + rot_dim),
           f"{what}: the cache {tuple(rows_cache.shape)} is not [pages, {PAGE_TOKENS}, {kv_rank + rot_dim}]")
     _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
     out = torch.empty((n, heads, kv_rank), dtype=F32, device=qa.device)
+    if rows_t is not None and not ctx.is_decode and latent_mfma_serves(rows_cache, kv_rank, rot_dim):
+        _need(table_t is not None and rows_t.dtype == BF16 and rows_t.dim() == 3 and rows_t.shape[1:] == (kv_rank, PAGE_TOKENS)
+              and table_t.shape == block_table.shape, f"{what}: the transposed copy is bfloat16 [pages, {kv_rank}, {PAGE_TOKENS}] with a page "
+              "table like the rows'")
+        library.call(latent_attention_lib(kv_rank, rot_dim), "palm_latent_attention_mfma", _stream(), _p(qa), _p(rows_cache), _p(rows_t),
+                     _p(block_table), _p(table_t), block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new),
+                     ctx.n_seqs, int(ctx.max_new), heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out))
+        return out
     library.call(mixers(), "palm_latent_attention", _stream(), _p(qa), _p(rows_cache), _code(rows_cache, what), _p(block_table),
                  block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
                  heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out))

@@ -9,7 +9,9 @@
 
 Keys and values are never expanded: q_plain goes through U_k,h once (a_h = U_k,h^T q_plain, kv_rank values), the scores
 are a_h . c_j + q_rot . r_j, the weighted sum is taken over the rows c_j, and U_v,h is applied to the sum.  All heads read
-the same rows.  The rotation's angles and the scores, weights and sums are 32-bit.
+the same rows.  The rotation's angles and the scores, weights and sums are 32-bit.  In the bfloat16 mode the cache keeps the
+latents a second time with the positions innermost, which is how the prompt kernel on the matrix cores reads them; single
+tokens and the float32 mode go through the exact kernel, which reads the rows alone.
 """
 from __future__ import annotations
 
@@ -52,19 +54,28 @@ class LatentAttention:
     @staticmethod
     def cache_needs(spec):
         p = spec.params
-        return [RowsNeed("latent", (int(p["kv_rank"]) + int(p["rot_dim"]),), None, int(p["window"]) if p.get("window") else None)]
+        window = int(p["window"]) if p.get("window") else None
+        # the rows, and the latents once more in bfloat16 for the prompt kernel on the matrix cores (a page of them is read
+        # there with the positions innermost: [kv_rank, 64] in the room of [64, kv_rank])
+        return [RowsNeed("latent", (int(p["kv_rank"]) + int(p["rot_dim"]),), None, window),
+                RowsNeed("latent_t", (int(p["kv_rank"]),), "bfloat16", window)]
 
     def forward(self, h, ctx):
         lc = ctx.layer_cache
         if lc is None or not lc.rows or "latent" not in lc.rows:
             raise RuntimeError("latent attention needs the rows of its layer; the step gave it no cache")
         view = lc.rows["latent"]
+        rows_t = table_t = None
+        if "latent_t" in lc.rows and ops.latent_mfma_serves(view.data, self.kv_rank, self.dr):
+            turned = lc.rows["latent_t"]
+            rows_t, table_t = turned.data.view(turned.data.shape[0], self.kv_rank, turned.data.shape[1]), turned.table_dev
         down = self.down(h)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         cq = ops.latent_prep(down, self.q_rank, self.q_rank, self.kv_rank, self.dr, self.q_norm_w, self.kv_norm_w, self.eps, cos, sin,
-                             view.data, view.table_dev, ctx, write_cache=lc.writes)
+                             view.data, view.table_dev, ctx, write_cache=lc.writes, rows_t=rows_t, table_t=table_t)
         qa = ops.latent_query(self.uq(cq), self.uk, cos, sin, self.nh, self.dk, self.dr, self.kv_rank)
-        o_lat = ops.latent_attention(qa, view.data, view.table_dev, ctx, self.nh, self.kv_rank, self.dr, self.scale, self.window)
+        o_lat = ops.latent_attention(qa, view.data, view.table_dev, ctx, self.nh, self.kv_rank, self.dr, self.scale, self.window,
+                                     rows_t=rows_t, table_t=table_t)
         gate = down[:, self.q_rank + self.kv_rank + self.dr:] if self.gated else None
         return self.out(ops.latent_output(o_lat, self.uv, gate, self.nh, self.kv_rank, self.dv, self.dtype))

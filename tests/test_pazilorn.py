@@ -52,8 +52,9 @@ def test_cache_needs_follow_the_run_order():
     spec = config_from_dict(S.CONFIGS["A"]).spec()
     needs = [cache_needs(spec.layers[c.layer]) for c in spec.order]
     assert needs[0] == needs[2] == [StateNeed("delta", (4, 16, 24)), StateNeed("delta_conv", (3, 2 * 2 * 16 + 4 * 24))]
-    assert needs[1] == needs[3] == [RowsNeed("latent", (48,), None, 37)]
-    assert cache_needs(config_from_dict(S.CONFIGS["C"]).spec().layers[0]) == [RowsNeed("latent", (74,), None, None)]
+    assert needs[1] == needs[3] == [RowsNeed("latent", (48,), None, 37), RowsNeed("latent_t", (40,), "bfloat16", 37)]
+    assert cache_needs(config_from_dict(S.CONFIGS["C"]).spec().layers[0]) == [RowsNeed("latent", (74,), None, None),
+                                                                              RowsNeed("latent_t", (70,), "bfloat16", None)]
 
 
 def test_ranks_come_from_the_tensors_where_config_json_has_none(tmp_path):
@@ -197,9 +198,10 @@ def assert_close(got, ref, dtype: str, what: str = "") -> None:
     """float32: 1e-4 of the logits' scale (and no less than 1e-4: some hundred steps of a 32-bit recurrence come to that on
     logits of several units), the gate that shows faults.  bfloat16: a row's root mean square error
     within a fifth of the logits' scale, all rows together within a twentieth, an element within three quarters; one row in
-    fifty (at least two) may be over the row gate, but never by more than the scale itself: which experts a token gets
-    turns on the rounding of the router's input when two logits lie close (one of five experts a token is a whole other
-    feed-forward then), with float32 twins exact."""
+    twenty-five (at least two) may be over the row gate, but never by more than the scale itself: which experts a token gets
+    turns on the rounding of the router's input when two logits lie close (with one of five experts a token, as one
+    configuration has it, that is a whole other feed-forward, and a rounding of one or two percent of the logits' spread
+    does it to some two tokens in a hundred), with float32 twins exact."""
     got = torch.as_tensor(got).double().cpu().reshape(ref.shape)
     assert torch.isfinite(got).all(), f"{what}: logits are not finite"
     err = (got - ref.double()).abs().reshape(-1, ref.shape[-1])
@@ -210,7 +212,7 @@ def assert_close(got, ref, dtype: str, what: str = "") -> None:
         return
     rows = err.pow(2).mean(-1).sqrt()
     over = rows > 0.2 * scale
-    assert int(over.sum()) <= max(2, rows.numel() // 50), (f"{what}: bfloat16 rms error over a fifth of {scale:.3e} in "
+    assert int(over.sum()) <= max(2, rows.numel() // 25), (f"{what}: bfloat16 rms error over a fifth of {scale:.3e} in "
                                                              f"{int(over.sum())} of {rows.numel()} rows, the worst {float(rows.max()):.3e} in row {int(rows.argmax())}")
     assert float(rows.max()) <= scale, f"{what}: bfloat16 rms error {float(rows.max()):.3e} in row {int(rows.argmax())} vs {scale:.3e}"
     rest = err[~over]
@@ -390,7 +392,8 @@ def _latent_plain(qa, rows, starts, counts, heads, R, scale, window):
 
 @gpu
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,R,dr,window", [(3, 40, 8, 37), (1, 96, 16, 70), (5, 70, 4, None), (2, 200, 32, 64), (2, 520, 64, 129)])
+@pytest.mark.parametrize("heads,R,dr,window", [(3, 40, 8, 37), (1, 96, 16, 70), (5, 70, 4, None), (2, 200, 32, 64), (2, 520, 64, 129),
+                                               (7, 256, 32, None), (5, 136, 16, 130)])
 def test_latent_attention_kernel_far_keys_page_borders_and_window_edges(dtype, heads, R, dr, window):
     """Two sequences through pages in a scrambled order, one as a prompt portion and one as a single token.  For chosen
     queries one key carries a large score: far back, on either side of a page border, the last key inside the window and
@@ -435,6 +438,19 @@ def test_latent_attention_kernel_far_keys_page_borders_and_window_edges(dtype, h
     want = _latent_plain(qa, [r[:-1] for r in rows], starts, counts, heads, R, 0.7, window)
     assert torch.isfinite(got).all()
     assert torch.allclose(got, want, atol=1e-4 if dtype == "float32" else 2e-2, rtol=1e-3 if dtype == "float32" else 2e-2), float((got - want).abs().max())
+    if dtype == "bfloat16" and ops.latent_mfma_serves(cache, R, dr):
+        # the prompt kernel on the matrix cores: the latents once more with the positions innermost, through pages in another
+        # scrambled order, NaN wherever the copy belongs to nobody
+        pages_t = [[3, 11, 0, 5, 7, 1], [2, 4, 12, 6]]
+        turned = torch.full((14, R, 64), float("nan"), dtype=td, device="cuda")
+        table_t = torch.full((3, 8), 13, dtype=torch.int32)
+        for b, pages in enumerate(pages_t):
+            table_t[b + 1, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+            for j in range(lens[b]):
+                turned[pages[j // 64], :, j % 64] = rows[b][j, :R].cuda()
+        fast = ops.latent_attention(qa.cuda(), cache, table, ctx, heads, R, dr, 0.7, window, rows_t=turned, table_t=table_t.cuda()).double().cpu()
+        assert torch.isfinite(fast).all()
+        assert torch.allclose(fast, want, atol=3e-2, rtol=3e-2), float((fast - want).abs().max())
     # the marked keys decide: a window one shorter, or the key outside seen, would change the marked rows by far more
     if window:
         other = _latent_plain(qa, [r[:-1] for r in rows], starts, counts, heads, R, 0.7, window - 1)
@@ -463,13 +479,18 @@ def test_latent_projections_around_the_attention(dtype):
     cos, sin = torch.cos(ang).float().cuda(), torch.sin(ang).float().cuda()
     cache = torch.zeros((4, 64, R + dr), dtype=td, device="cuda")
     table = torch.tensor([[2, 1], [0, 3], [3, 3]], dtype=torch.int32, device="cuda")
-    cq = ops.latent_prep(down.cuda(), Q, Q, R, dr, wq.cuda(), wk.cuda(), 1e-5, cos, sin, cache, table, ctx)
+    turned = torch.zeros((4, R, 64), dtype=torch.bfloat16, device="cuda")
+    table_t = torch.tensor([[1, 3], [2, 0], [3, 3]], dtype=torch.int32, device="cuda")
+    cq = ops.latent_prep(down.cuda(), Q, Q, R, dr, wq.cuda(), wk.cuda(), 1e-5, cos, sin, cache, table, ctx, rows_t=turned, table_t=table_t)
     dd = down.double()
     assert torch.allclose(cq.double().cpu(), P.rms_norm(dd[:, :Q], wq.double(), 1e-5), **tol)
     want_rows = torch.cat([P.rms_norm(dd[:, Q:Q + R], wk.double(), 1e-5), P.rotate(dd[:, Q + R:Q + R + dr], pos, rot)], 1)
     where = [(1, 60 + i - 64) if 60 + i >= 64 else (2, 60 + i) for i in range(8)] + [(0, i) for i in range(3)]
     got_rows = torch.stack([cache[p, j] for p, j in where]).double().cpu()
     assert torch.allclose(got_rows, want_rows, **tol)
+    where_t = [(3, 60 + i - 64) if 60 + i >= 64 else (1, 60 + i) for i in range(8)] + [(2, i) for i in range(3)]
+    got_t = torch.stack([turned[p, :, j] for p, j in where_t]).double().cpu()
+    assert torch.allclose(got_t, want_rows[:, :R], atol=0.03, rtol=0.02)
     q = torch.randn(n, H * (d + dr), generator=g).to(td)
     uk = (torch.randn(H * d, R, generator=g) * 0.3).to(td)
     qa = ops.latent_query(q.cuda(), uk.cuda(), cos, sin, H, d, dr, R).double().cpu()
