@@ -11,7 +11,9 @@
 // bfloat16 for the second product, whose sums are 32-bit again.
 //
 // rows [pages, 64, kv_rank + rot_dim]: the keys; rows_t [pages, kv_rank, 64]: the latents once more, positions innermost.
-// The two have page tables of their own.  q: float32 [n, heads, kv_rank + rot_dim]; out: float32 [n, heads, kv_rank].
+// The two have page tables of their own.  q: float32 [n, heads, kv_rank + rot_dim]; out: float32 [n, heads, kv_rank], or,
+// with the value matrices uv [heads * vdim, kv_rank] (and the heads' gates before their sigmoid), out_rows bfloat16
+// [n, heads * vdim]: head h's sums through U_v,h times sigmoid(gate_h), made from the registers that hold the sums.
 #include "mfma.h"
 
 #ifndef PALM_LAT_KK
@@ -47,7 +49,8 @@ __global__ __launch_bounds__(WAVE) void latent_attention_mfma_kernel(
     const float* __restrict__ q, const bf16_t* __restrict__ rows, const bf16_t* __restrict__ rows_t,
     const int* __restrict__ block_table, const int* __restrict__ block_table_t, int max_pages,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_new,
-    const int* __restrict__ cu_new, int heads, int kv_rank, int rot_dim, float scale, int window, float* __restrict__ out) {
+    const int* __restrict__ cu_new, int heads, int kv_rank, int rot_dim, float scale, int window, float* __restrict__ out,
+    const bf16_t* __restrict__ uv, const bf16_t* __restrict__ gate, int gate_stride, int vdim, bf16_t* __restrict__ out_rows) {
     const int h0 = blockIdx.y * HT, b = blockIdx.z;
     const int n_new = seq_new[b];
     const int lane = threadIdx.x;
@@ -173,6 +176,47 @@ __global__ __launch_bounds__(WAVE) void latent_attention_mfma_kernel(
         l[t] += __shfl_xor(l[t], 16, WAVE);
         l[t] += __shfl_xor(l[t], 32, WAVE);
     }
+    if (uv) {
+        // The value matrix in the same kernel: out^T [vdim, 16 queries] = U_v,h [vdim, kv_rank] (O^T / l).  The sums a lane
+        // holds (latent dimensions 16 vt + 4 g + i of query r) are, two tiles at a time, the B operand of a step over 32
+        // latent dimensions; the A operand takes the same dimensions of a row of U_v,h.  Then the head's gate.
+        constexpr int VP = (VT + 1) / 2;
+#pragma unroll
+        for (int t = 0; t < HT; ++t) {
+            const int h = min(h0 + t, heads - 1);
+            const float f = 1.0f / l[t];
+            bf16x8 of[VP];
+#pragma unroll
+            for (int m = 0; m < VP; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    of[m][i] = (__bf16)(acc[t][2 * m][i] * f);
+                    of[m][4 + i] = (__bf16)(2 * m + 1 < VT ? acc[t][min(2 * m + 1, VT - 1)][i] * f : 0.f);
+                }
+            const float gt = gate ? 1.0f / (1.0f + expf(-to_float(gate[((size_t)cu_new[b] + qi) * gate_stride + h]))) : 1.0f;
+            for (int j0 = 0; j0 < vdim; j0 += 16) {
+                const bf16_t* wr = uv + ((size_t)h * vdim + min(j0 + r, vdim - 1)) * kv_rank;
+                f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int m = 0; m < VP; ++m) {
+                    const int k0 = 32 * m + 4 * g, k1 = 32 * m + 16 + 4 * g;          // four dimensions each, inside the latent or beyond it
+                    const uint2 lo = *reinterpret_cast<const uint2*>(wr + min(k0, kv_rank - 4));
+                    const uint2 hi = *reinterpret_cast<const uint2*>(wr + min(k1, kv_rank - 4));
+                    const uint4 both = make_uint4(k0 < kv_rank ? lo.x : 0u, k0 < kv_rank ? lo.y : 0u, k1 < kv_rank ? hi.x : 0u, k1 < kv_rank ? hi.y : 0u);
+                    o = mfma_16x16x32(__builtin_bit_cast(bf16x8, both), of[m], o);
+                }
+                // lane (r, g) holds output dimensions j0 + 4 g + i of query r
+                const int j = j0 + 4 * g;
+                if (q0 + r < n_new && h0 + t < heads && j < vdim) {                   // vdim is a multiple of four
+                    uint2 w;
+                    w.x = (uint32_t)f32_to_bf16(o[0] * gt).bits | ((uint32_t)f32_to_bf16(o[1] * gt).bits << 16);
+                    w.y = (uint32_t)f32_to_bf16(o[2] * gt).bits | ((uint32_t)f32_to_bf16(o[3] * gt).bits << 16);
+                    *reinterpret_cast<uint2*>(out_rows + (((size_t)cu_new[b] + qi) * heads + h0 + t) * vdim + j) = w;
+                }
+            }
+        }
+        return;
+    }
     if (q0 + r >= n_new) return;
 #pragma unroll
     for (int t = 0; t < HT; ++t) {
@@ -191,7 +235,8 @@ __global__ __launch_bounds__(WAVE) void latent_attention_mfma_kernel(
 PALM_API int palm_latent_attention_mfma(hipStream_t stream, const float* q, const void* rows, const void* rows_t,
                                         const int* block_table, const int* block_table_t, int max_pages, const int* seq_slot,
                                         const int* seq_start, const int* seq_new, const int* cu_new, int n_seqs, int max_new,
-                                        int heads, int kv_rank, int rot_dim, float scale, int window, float* out) {
+                                        int heads, int kv_rank, int rot_dim, float scale, int window, float* out, const void* uv,
+                                        const void* gate, int gate_stride, int vdim, void* out_rows) {
     PALM_CHECK(n_seqs >= 0 && max_new >= 0 && heads > 0 && kv_rank > 0 && rot_dim >= 0, "latent_attention_mfma: seqs=%d max_new=%d heads=%d "
                "kv_rank=%d rot_dim=%d", n_seqs, max_new, heads, kv_rank, rot_dim);
     const int dk = kv_rank + rot_dim;
@@ -200,12 +245,15 @@ PALM_API int palm_latent_attention_mfma(hipStream_t stream, const float* q, cons
     PALM_CHECK(kv_rank % 8 == 0 && kv_rank <= VT * 16 && kv_rank > (VT - 1) * 16, "latent_attention_mfma: built for latents of %d..%d in "
                "steps of 8, not %d", (VT - 1) * 16 + 8, VT * 16, kv_rank);
     PALM_CHECK(window >= 0 && max_pages > 0, "latent_attention_mfma: window %d, max_pages %d", window, max_pages);
+    PALM_CHECK(uv ? (out_rows && vdim > 0 && vdim % 4 == 0) : out != nullptr, "latent_attention_mfma: either room for the latent sums, or the "
+               "value matrix with room for rows of a value size that is a multiple of four (%d)", vdim);
     if (n_seqs == 0 || max_new == 0) return 0;
     PALM_CHECK(heads <= 65535 * HT && n_seqs <= 65535, "latent_attention_mfma: %d heads / %d sequences are more than one launch takes", heads, n_seqs);
     dim3 grid((max_new + 15) / 16, (heads + HT - 1) / HT, n_seqs);
     latent_attention_mfma_kernel<<<grid, WAVE, 0, stream>>>(q, (const bf16_t*)rows, (const bf16_t*)rows_t, block_table, block_table_t,
                                                            max_pages, seq_slot, seq_start, seq_new, cu_new, heads, kv_rank, rot_dim, scale,
-                                                           window, out);
+                                                           window, out, (const bf16_t*)uv, (const bf16_t*)gate, gate_stride, vdim,
+                                                           (bf16_t*)out_rows);
     PALM_LAUNCHED();
     return 0;
 }

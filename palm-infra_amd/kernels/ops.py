@@ -1195,7 +1195,7 @@ def latent_query(q: torch.Tensor, uk: torch.Tensor, cos, sin, heads: int, dim: i
 
 
 _LATENT_MFMA_SIGNATURE = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                          c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]
+                          c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
 _latent_libs: dict = {}
 LATENT_MFMA_MAX_ROW, LATENT_MFMA_MAX_RANK = 640, 512
 
@@ -1241,11 +1241,41 @@ def latent_attention(qa: torch.Tensor, rows_cache: torch.Tensor, block_table: to
               "table like the rows'")
         library.call(latent_attention_lib(kv_rank, rot_dim), "palm_latent_attention_mfma", _stream(), _p(qa), _p(rows_cache), _p(rows_t),
                      _p(block_table), _p(table_t), block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new),
-                     ctx.n_seqs, int(ctx.max_new), heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out))
+                     ctx.n_seqs, int(ctx.max_new), heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out), None, None, 0, 0, None)
         return out
     library.call(mixers(), "palm_latent_attention", _stream(), _p(qa), _p(rows_cache), _code(rows_cache, what), _p(block_table),
                  block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new), ctx.n_seqs, int(ctx.max_new),
                  heads, kv_rank, rot_dim, float(scale), int(window or 0), _p(out))
+    return out
+
+
+def latent_fused_serves(qa: torch.Tensor, rows_cache: torch.Tensor, rows_t, uv: torch.Tensor, ctx, kv_rank: int, rot_dim: int, vdim: int) -> bool:
+    """Whether the prompt kernel on the matrix cores also applies the value matrices: a prompt (or a portion) in bfloat16 with
+    the transposed copy of the latents at hand, bfloat16 matrices, a value size that is a multiple of four."""
+    return (rows_t is not None and not ctx.is_decode and uv.dtype == BF16 and vdim % 4 == 0 and latent_mfma_serves(rows_cache, kv_rank, rot_dim))
+
+
+def latent_attention_fused(qa: torch.Tensor, rows_cache: torch.Tensor, block_table: torch.Tensor, ctx, heads: int, kv_rank: int,
+                           rot_dim: int, scale: float, window: int | None, rows_t: torch.Tensor, table_t: torch.Tensor, uv: torch.Tensor,
+                           gate: torch.Tensor | None, vdim: int) -> torch.Tensor:
+    """``latent_attention`` on the matrix cores and ``latent_output`` in one kernel: bfloat16 [n, heads * vdim]."""
+    what = "latent_attention_fused"
+    _dev(what, qa, rows_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new, rows_t, table_t, uv)
+    _i32(what, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new, table_t)
+    n = qa.shape[0]
+    _need(latent_fused_serves(qa, rows_cache, rows_t, uv, ctx, kv_rank, rot_dim, vdim), f"{what}: a prompt in bfloat16 with sizes the kernel takes")
+    _need(qa.shape == (n, heads, kv_rank + rot_dim) and qa.dtype == F32 and n == ctx.n_tokens, f"{what}: queries {tuple(qa.shape)} {qa.dtype}")
+    _need(rows_cache.dim() == 3 and rows_cache.shape[1:] == (PAGE_TOKENS, kv_rank + rot_dim) and rows_t.dtype == BF16 and rows_t.dim() == 3
+          and rows_t.shape[1:] == (kv_rank, PAGE_TOKENS) and block_table.dim() == 2 and table_t.shape == block_table.shape,
+          f"{what}: the cache {tuple(rows_cache.shape)}, its transposed copy {tuple(rows_t.shape)}, page tables {tuple(block_table.shape)}")
+    _need(uv.shape == (heads * vdim, kv_rank), f"{what}: value matrix {tuple(uv.shape)} for {heads} heads of {vdim} over a latent of {kv_rank}")
+    _need(gate is None or (gate.is_cuda and gate.shape == (n, heads) and gate.dtype == BF16 and (n == 0 or gate.stride(1) == 1)),
+          f"{what}: the gate is bfloat16 [{n}, {heads}] with contiguous rows")
+    out = torch.empty((n, heads * vdim), dtype=BF16, device=qa.device)
+    library.call(latent_attention_lib(kv_rank, rot_dim), "palm_latent_attention_mfma", _stream(), _p(qa), _p(rows_cache), _p(rows_t),
+                 _p(block_table), _p(table_t), block_table.shape[1], _p(ctx.seq_slot), _p(ctx.seq_start), _p(ctx.seq_new), _p(ctx.cu_new),
+                 ctx.n_seqs, int(ctx.max_new), heads, kv_rank, rot_dim, float(scale), int(window or 0), None, _p(uv), _p(gate),
+                 gate.stride(0) if gate is not None else 0, vdim, _p(out))
     return out
 
 

@@ -75,7 +75,12 @@ class LatentAttention:
         cq = ops.latent_prep(down, self.q_rank, self.q_rank, self.kv_rank, self.dr, self.q_norm_w, self.kv_norm_w, self.eps, cos, sin,
                              view.data, view.table_dev, ctx, write_cache=lc.writes, rows_t=rows_t, table_t=table_t)
         qa = ops.latent_query(self.uq(cq), self.uk, cos, sin, self.nh, self.dk, self.dr, self.kv_rank)
+        gate = down[:, self.q_rank + self.kv_rank + self.dr:] if self.gated else None
+        if ops.latent_fused_serves(qa, view.data, rows_t, self.uv, ctx, self.kv_rank, self.dr, self.dv):
+            # a prompt on the matrix cores: the value matrices and the gates ride in the attention kernel
+            o = ops.latent_attention_fused(qa, view.data, view.table_dev, ctx, self.nh, self.kv_rank, self.dr, self.scale, self.window,
+                                           rows_t, table_t, self.uv, gate, self.dv)
+            return self.out(o)
         o_lat = ops.latent_attention(qa, view.data, view.table_dev, ctx, self.nh, self.kv_rank, self.dr, self.scale, self.window,
                                      rows_t=rows_t, table_t=table_t)
-        gate = down[:, self.q_rank + self.kv_rank + self.dr:] if self.gated else None
         return self.out(ops.latent_output(o_lat, self.uv, gate, self.nh, self.kv_rank, self.dv, self.dtype))

@@ -451,6 +451,15 @@ def test_latent_attention_kernel_far_keys_page_borders_and_window_edges(dtype, h
         fast = ops.latent_attention(qa.cuda(), cache, table, ctx, heads, R, dr, 0.7, window, rows_t=turned, table_t=table_t.cuda()).double().cpu()
         assert torch.isfinite(fast).all()
         assert torch.allclose(fast, want, atol=3e-2, rtol=3e-2), float((fast - want).abs().max())
+        # and with the value matrices and the heads' gates in the same kernel (value sizes that fill no tile of 16 too)
+        for dv in (20, 72):
+            uv = (torch.randn(heads * dv, R, generator=g) * 0.2).to(td)
+            gate = torch.randn(n, heads + 3, generator=g).to(td)
+            fused = ops.latent_attention_fused(qa.cuda(), cache, table, ctx, heads, R, dr, 0.7, window, turned, table_t.cuda(), uv.cuda(),
+                                               gate.cuda()[:, 3:], dv).double().cpu()
+            rows_out = torch.einsum("thr,hvr->thv", want, uv.double().reshape(heads, dv, R)) * torch.sigmoid(gate.double()[:, 3:]).unsqueeze(-1)
+            assert torch.isfinite(fused).all()
+            assert torch.allclose(fused, rows_out.reshape(n, heads * dv), atol=4e-2, rtol=4e-2), float((fused - rows_out.reshape(n, heads * dv)).abs().max())
     # the marked keys decide: a window one shorter, or the key outside seen, would change the marked rows by far more
     if window:
         other = _latent_plain(qa, [r[:-1] for r in rows], starts, counts, heads, R, 0.7, window - 1)
