@@ -49,7 +49,7 @@ ATTENTION_SOURCES = ["attention_mfma.hip"]
 DIFF_ATTENTION_SOURCES = ["attention_diff_mfma.hip"]
 LATENT_ATTENTION_SOURCES = ["latent_attention_mfma.hip"]
 MIXER_SOURCES = ["stream.hip", "retention.hip", "mamba.hip", "attention_diff.hip", "residual_scaled.hip", "delta_rule.hip",
-                 "latent_attention.hip", "moe.hip"]
+                 "latent_attention.hip", "moe.hip", "moe_grouped.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
 

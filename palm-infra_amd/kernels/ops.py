@@ -791,6 +791,9 @@ _MIXER_SIGNATURES = {
     "palm_moe_route": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
     "palm_moe_experts": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                          c_void_p, c_void_p],
+    "palm_moe_tile_tokens": [],
+    "palm_moe_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                         c_void_p, c_void_p],
     "palm_gather_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "palm_scatter_add": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -1325,6 +1328,37 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chos
     out = torch.empty((n, width), dtype=F32, device=h.device)
     library.call(mixers(), "palm_moe_experts", _stream(), _p(h), _code(h, what), _p(gate_up), _p(down), _code(gate_up, what + " weights"),
                  _p(chosen), _p(weight), n, top, width, ff, _p(mid), _p(out))
+    return out
+
+
+def moe_grouped_serves(h: torch.Tensor, gate_up: torch.Tensor, ff: int) -> bool:
+    """The grouped products on the matrix cores take bfloat16 rows and weights whose sizes are multiples of eight."""
+    return h.dtype == BF16 and gate_up.dtype == BF16 and h.shape[1] % 8 == 0 and ff % 8 == 0
+
+
+def moe_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, ff: int) -> torch.Tensor:
+    """Every row through its chosen experts, for many rows, planned on the device: the (row, choice) pairs grouped by expert,
+    two grouped products on the matrix cores, the weighted sum in the order of the choices.  Shapes as ``moe_experts``;
+    returns float32 [n, width]."""
+    what = "moe_grouped"
+    _dev(what, h, gate_up, down, chosen, weight)
+    _i32(what, chosen)
+    n, width = h.shape
+    top = chosen.shape[1]
+    _need(moe_grouped_serves(h, gate_up, ff), f"{what}: bfloat16 rows and weights, sizes in multiples of eight")
+    _need(gate_up.dim() == 2 and gate_up.shape[1] == width and gate_up.shape[0] % (2 * ff) == 0 and down.shape == (gate_up.shape[0] // (2 * ff) * width, ff)
+          and down.dtype == BF16, f"{what}: gate/up {tuple(gate_up.shape)}, down {tuple(down.shape)} for width {width}, inner size {ff}")
+    _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == F32, f"{what}: choices {tuple(chosen.shape)}, weights {tuple(weight.shape)}")
+    experts = gate_up.shape[0] // (2 * ff)
+    tile = mixers().palm_moe_tile_tokens()
+    max_tiles = (n * top + tile - 1) // tile + experts
+    slots = max_tiles * tile
+    plan = torch.empty((2 * experts + 1 + max_tiles + slots + n * top,), dtype=torch.int32, device=h.device)
+    mid = torch.empty((slots, ff), dtype=BF16, device=h.device)
+    y = torch.empty((slots, width), dtype=BF16, device=h.device)
+    out = torch.empty((n, width), dtype=F32, device=h.device)
+    library.call(mixers(), "palm_moe_grouped", _stream(), _p(h), _p(gate_up), _p(down), _p(chosen), _p(weight), n, top, experts, width, ff,
+                 _p(plan), _p(mid), _p(y), _p(out))
     return out
 
 

@@ -7,7 +7,9 @@ joined into one [2I, H] product (models/qwen3.py:276-287; kernels/elementwise.cp
 logits W_r h + b are 32-bit, the ``top`` largest choose the experts, their weights are the softmax over those logits
 alone, and the output is the weighted sum of the chosen experts' outputs.  A step of few rows (a decode step) reads each
 (token, choice)'s expert in the kernel, nothing planned on the host (and so it can be recorded); a prompt's (token,
-choice) pairs are grouped by expert on the host and every expert's rows go through its two products together.
+choice) pairs are grouped by expert on the device and all experts' rows go through two grouped products on the matrix
+cores (bfloat16); in the float32 mode, and for sizes those do not take, the host groups the pairs and every expert's
+rows go through its two products as ``Linear`` makes them.
 
 ``dense``: down(act(up(h))) with an activation chosen by name.  ``xielu`` has two learned numbers p, q (tensor
 ``activation``, float32 [2]): for z > 0, softplus(p) z^2 + z/2; for z <= 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
@@ -94,6 +96,8 @@ class RoutedGatedSiluFeedForward:
         chosen, weight = ops.moe_route(self.router(h, out_dtype=torch.float32), self.top)
         if h.shape[0] <= self.DIRECT_ROWS:
             return ops.moe_experts(h, self.gate_up, self.down, chosen, weight, self.inter)
+        if ops.moe_grouped_serves(h, self.gate_up, self.inter):
+            return ops.moe_grouped(h, self.gate_up, self.down, chosen, weight, self.inter)
         # group the (token, choice) pairs by expert; within an expert in the order of the tokens
         flat = chosen.to("cpu").numpy().reshape(-1)
         order = np.argsort(flat, kind="stable").astype(np.int32)
