@@ -358,11 +358,14 @@ def _mixer_rooflines(raw: dict, tokens: int, batch: int, context: int) -> dict:
                 w = m["mask"]["size"] if m.get("mask") else tokens
                 seen = sum(min(p + 1, w) for p in range(tokens))
                 row = m["kv_rank"] + m["rot_dim"]
-                out["palm_latent_attention"] = (2.0 * m["heads"] * (row + m["kv_rank"]) * seen, mfma,
-                                                2.0 * batch * min(context, w) * row, hbm)
+                flops = 2.0 * m["heads"] * (row + m["kv_rank"]) * seen
+                out["palm_latent_attention"] = (flops, mfma, 2.0 * batch * min(context, w) * row, hbm)
+                # the prompt kernel also applies the value matrices
+                out["palm_latent_attention_mfma"] = (flops + 2.0 * tokens * m["heads"] * m["kv_rank"] * m["vdim"], mfma, None, None)
             if layer.get("mlp") and layer["mlp"].get("kind") == "moe" and "palm_moe_experts" not in out:
                 f = layer["mlp"]
                 out["palm_moe_experts"] = (None, None, 2.0 * batch * f["router"]["top"] * 3 * f["expert"]["ff"] * raw["width"], hbm)
+                out["palm_moe_grouped"] = (2.0 * tokens * f["router"]["top"] * 3 * f["expert"]["ff"] * raw["width"], mfma, None, None)
     else:
         nh, nkv, hd = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
         out["palm_attention_prefill"] = (4.0 * nh * hd * pairs, mfma, None, None)
