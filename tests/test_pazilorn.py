@@ -346,7 +346,7 @@ def _delta_plain(c, heads, kv, dim, vdim, eps, drop_first=False):
 
 @gpu
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv,dim,vdim", [(2, 1, 12, 20), (3, 3, 40, 72), (1, 1, 96, 130), (2, 2, 130, 64)])
+@pytest.mark.parametrize("heads,kv,dim,vdim", [(2, 1, 12, 20), (3, 3, 40, 72), (1, 1, 96, 130), (2, 2, 130, 64), (2, 2, 32, 320)])
 def test_delta_rule_kernel_keeps_a_far_write_whole_and_in_portions(dtype, heads, kv, dim, vdim):
     """Whole, in portions down to two tokens and single tokens, and cut by the kernel into chunks that run side by side (of
     a size given here, 0 for none, or of its own choice): the outputs and the state left behind."""
