@@ -250,8 +250,12 @@ class PazilornConfig:
                      "gate_up": joined(gu_names, gu_shapes, "matrix", ("normal", 0.0, 0.08)),
                      "down": joined([f"{p}mlp.e{e}.down" for e in range(E)], [(W, F)] * E, "matrix", ("normal", 0.0, 0.08))})
                 parts["feed_forward_out_norm"] = norm(p + "norm2b")
+            # a checkpoint that holds the second pair of norms for a layer without a feed-forward: bound, and not used
+            spare = {}
+            if layer["mlp"] is None and tensor_names is not None:
+                spare = {f"spare_{n}": tensor(p + n, (W,), "vector", _NORM_INIT) for n in ("norm2", "norm2b") if p + n in set(tensor_names)}
             index[i] = len(layers)
-            layers.append(PartSpec("block", "sandwich", {"hidden_size": W, "residual_gain": self.residual_mult}, {}, parts))
+            layers.append(PartSpec("block", "sandwich", {"hidden_size": W, "residual_gain": self.residual_mult}, spare, parts))
         order = tuple(LayerCall(index[self._source(self.layers, i)]) for i in range(len(self.layers)))
 
         table = tensor("embed", (V, W), "table", ("normal", 0.0, 0.05))

@@ -46,6 +46,15 @@ def test_spec_names_every_tensor_and_borrowed_layers_have_none():
     assert "head" not in names                                             # the head is the table itself
 
 
+def test_norms_of_a_feed_forward_that_is_not_there_are_bound_and_not_missed():
+    cfg = config_from_dict(S.CONFIGS["A"])
+    names = list(cfg.spec().expected_tensors())
+    assert "l1.norm2" not in names
+    with_spares = cfg.spec(names + ["l1.norm2", "l1.norm2b"]).expected_tensors()
+    assert with_spares["l1.norm2"][0] == (64,) and with_spares["l1.norm2b"][0] == (64,) and len(with_spares) == len(names) + 2
+    assert set(cfg.spec(names).expected_tensors()) == set(names)
+
+
 def test_cache_needs_follow_the_run_order():
     from palm_infra_amd.cache import RowsNeed, StateNeed
     from palm_infra_amd.parts import cache_needs
@@ -565,6 +574,25 @@ def test_each_request_alone_and_whole(tmp_path_factory, name, dtype):
         eng.close(slot)
         assert_close(got, reference(tmp_path_factory, name, dtype, ids), dtype, f"{name} whole {len(ids)}")
     eng.cache.check()
+
+
+@gpu
+def test_a_checkpoint_with_norms_for_a_feed_forward_that_is_not_there(tmp_path):
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import write_safetensors
+    raw = raw_of("A")
+    tensors = S.sharpened_tensors(raw, 7, "float32")
+    tensors["l1.norm2"] = torch.full((64,), 3.0)
+    tensors["l1.norm2b"] = torch.full((64,), -2.0)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    eng = Engine.from_dir(tmp_path, dtype="float32", max_tokens=256)
+    ids = S.prompts(raw, [40], seed=12)[0]
+    slot = eng.open()
+    got = eng.step([StepEntry(slot, ids, list(range(len(ids))))])
+    eng.close(slot)
+    cfg, w = P.read_model(tmp_path)
+    assert_close(got, P.forward(cfg, w, ids), "float32", "spare norms")
 
 
 @gpu
